@@ -85,10 +85,19 @@ class CacheManager:
         self.device = torch.device(device)
         self.dtype = dtype
         self.needs = list(needs)
-        self.groups: List[_Group] = []
-        self.group_of_entry: Dict[int, int] = {}
-        by_window: Dict[int, int] = {}
+        # A cache entry may need several things at once (a mixer that runs an attention beside a recurrence, a
+        # recurrence with two states): its need is then a tuple, each member is kept under the key (entry, index),
+        # and the entry's view is the tuple of the members' views.  A plain entry's key is the entry itself.
+        self._members: List[tuple] = []
         for e, need in enumerate(self.needs):
+            if isinstance(need, (tuple, list)):
+                self._members += [((e, j), n) for j, n in enumerate(need)]
+            else:
+                self._members.append((e, need))
+        self.groups: List[_Group] = []
+        self.group_of_entry: Dict[object, int] = {}
+        by_window: Dict[int, int] = {}
+        for e, need in self._members:
             if isinstance(need, PagedKV):
                 if need.window not in by_window:
                     n = (num_pages_per_group or {}).get(need.window, num_pages)
@@ -98,10 +107,10 @@ class CacheManager:
                 self.groups[g].entries.append(e)
                 self.group_of_entry[e] = g
         # data plane
-        self.k: Dict[int, torch.Tensor] = {}
-        self.v: Dict[int, torch.Tensor] = {}
-        self.state: Dict[int, torch.Tensor] = {}
-        for e, need in enumerate(self.needs):
+        self.k: Dict[object, torch.Tensor] = {}
+        self.v: Dict[object, torch.Tensor] = {}
+        self.state: Dict[object, torch.Tensor] = {}
+        for e, need in self._members:
             if isinstance(need, PagedKV):
                 n = self.groups[self.group_of_entry[e]].pool.num_pages
                 # keys [pages, nkv, page, d]; values transposed [pages, nkv, d, page], so that the
@@ -133,7 +142,7 @@ class CacheManager:
     # ---- sizes ----------------------------------------------------------------------------------
     def bytes_per_token(self) -> int:
         total = 0
-        for e, need in enumerate(self.needs):
+        for e, need in self._members:
             if isinstance(need, PagedKV):
                 total += 2 * need.num_kv_heads * need.head_dim * self.k[e].element_size()
         return total
@@ -354,6 +363,11 @@ class CacheManager:
     # ---- what a layer sees --------------------------------------------------------------------
     def view(self, entry: int, batch, writes: bool):
         need = self.needs[entry]
+        if isinstance(need, (tuple, list)):
+            return tuple(self._view((entry, j), n, batch, writes) for j, n in enumerate(need))
+        return self._view(entry, need, batch, writes)
+
+    def _view(self, entry, need, batch, writes: bool):
         if isinstance(need, PagedKV):
             g = self.group_of_entry[entry]
             return KVView(self.k[entry], self.v[entry], self.page_size, batch.block_tables[g],

@@ -1,4 +1,5 @@
-"""What a mixer asks of the cache manager for one cache entry."""
+"""What a mixer asks of the cache manager for one cache entry: one of the needs below, or a tuple of them (the
+mixer's view of the cache is then the tuple of their views)."""
 from __future__ import annotations
 
 from dataclasses import dataclass

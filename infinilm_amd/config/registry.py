@@ -2,7 +2,7 @@
 
 Role of csrc/models/models_registry.{hpp,cpp} and model_factory.cpp:6-26 in the reference: a name
 from config.json selects how the configuration is completed and which model is built.  Lookup
-goes by `architectures[0]` first, then by `model_type`.
+goes by `architectures[0]` first, then by `model_type`, then by `architecture`.
 """
 from __future__ import annotations
 
@@ -42,7 +42,7 @@ def resolve_architecture(raw: Dict[str, Any]) -> Architecture:
     archs = raw.get("architectures") or []
     if isinstance(archs, str):
         archs = [archs]
-    for n in list(archs) + [raw.get("model_type")]:
+    for n in list(archs) + [raw.get("model_type"), raw.get("architecture")]:   # (`architecture`: a single name)
         if n is None:
             continue
         tried.append(str(n))

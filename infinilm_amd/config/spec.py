@@ -45,6 +45,8 @@ class HeadSpec:
     name: str = "lm_head"
     scale: float = 1.0
     tie_to_embedding_when_missing: bool = True
+    # the head has no tensor of its own in any checkpoint: it reads the embedding's table (`name` is then unused)
+    always_tied: bool = False
     kind: str = "linear"
     params: Dict[str, Any] = field(default_factory=dict)
 

@@ -62,7 +62,7 @@ __global__ void __launch_bounds__(64)
 attn_basic_kernel(T* __restrict__ out, float* __restrict__ ws, const T* __restrict__ q, const T* __restrict__ kc,
                   const T* __restrict__ vc, const int* __restrict__ block_tables,
                   const int* __restrict__ seg, const int* __restrict__ pos, int nh, int nkv, int d,
-                  int page, int max_blocks, int q_stride, int out_stride, float scale, int window) {
+                  int page, int max_blocks, int q_stride, int out_stride, float scale, int window, float softcap) {
     extern __shared__ float smem[];
     float* qs = smem;      // d
     float* ps = smem + d;  // 64
@@ -106,6 +106,7 @@ attn_basic_kernel(T* __restrict__ out, float* __restrict__ ws, const T* __restri
                     for (int i = 0; i < d; ++i) dot = fmaf(qs[i], to_f32(krow[i]), dot);
                 }
                 s = dot * scale;
+                if (softcap > 0.f) s = softcap * tanhf(s / softcap);   // scores capped smoothly at +-softcap
             }
             const float m_new = fmaxf(m, wave_max(s));
             const float pj = valid ? expf(s - m_new) : 0.f;
@@ -212,7 +213,7 @@ extern "C" int ilm_attn_basic_chunk() { return AB_CHUNK; }
 extern "C" int ilm_attn_basic(void* out, void* ws, int nchunks, const void* q, const void* kc, const void* vc,
                               const void* block_tables, const void* seg, const void* pos, int T_,
                               int nh, int nkv, int d, int page, int max_blocks, int q_stride,
-                              int out_stride, float scale, int window, int dtype,
+                              int out_stride, float scale, int window, int dtype, float softcap,
                               hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && nh > 0 && nkv > 0 && d > 0 && page > 0 && max_blocks > 0, "attn_basic: bad sizes");
     ILM_REQUIRE(nh % nkv == 0, "attn_basic: %d query heads do not divide into %d groups", nh, nkv);
@@ -226,7 +227,7 @@ extern "C" int ilm_attn_basic(void* out, void* ws, int nchunks, const void* q, c
 #define AB_LAUNCH(T_, VEC_)                                                                                             \
     attn_basic_kernel<T_, VEC_><<<grid, 64, shm, stream>>>(                                                             \
         (T_*)out, (float*)ws, (const T_*)q, (const T_*)kc, (const T_*)vc, (const int*)block_tables, (const int*)seg,    \
-        (const int*)pos, nh, nkv, d, page, max_blocks, q_stride, out_stride, scale, window)
+        (const int*)pos, nh, nkv, d, page, max_blocks, q_stride, out_stride, scale, window, softcap)
     if (dtype == ILM_DTYPE_F32) {
         if (vec) AB_LAUNCH(float, true); else AB_LAUNCH(float, false);
     } else {

@@ -46,7 +46,7 @@ __global__ void __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(DT <= 8
 attn_f32_kernel(float* __restrict__ out, float* __restrict__ ws, const float* __restrict__ qp, const float* __restrict__ kc,
                 const float* __restrict__ vc, const int* __restrict__ block_tables, const int* __restrict__ seg,
                 const int* __restrict__ pos, int nh, int nkv, int nsub, int page, int max_blocks, int q_stride,
-                int out_stride, float scale, int window) {
+                int out_stride, float scale, int window, float softcap) {
     constexpr int d = DT * 16;
     // tiles of keys (and of values) in flight: two, or one where the running result of the wave that walks all
     // chunks leaves no registers for the second (another wave of the SIMD then covers the wait)
@@ -112,7 +112,11 @@ attn_f32_kernel(float* __restrict__ out, float* __restrict__ ws, const float* __
             }
             const int key0 = c * FA_CHUNK + kt * 16 + 4 * q;   // element e is the score of key key0 + e
 #pragma unroll
-            for (int e = 0; e < 4; ++e) S[kt][e] = (key0 + e >= k_lo && key0 + e <= k_hi) ? s[e] * scale : -INFINITY;
+            for (int e = 0; e < 4; ++e) {
+                float sc = s[e] * scale;
+                if (softcap > 0.f) sc = softcap * tanhf(sc / softcap);   // scores capped smoothly at +-softcap
+                S[kt][e] = (key0 + e >= k_lo && key0 + e <= k_hi) ? sc : -INFINITY;
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
 #undef FA_LOAD_K
@@ -259,7 +263,7 @@ extern "C" int ilm_attn_f32_ws_row(int d) { return d + FA_WS_PAD; }
 // nchunks >= ceil((largest position + 1) / ilm_attn_f32_chunk()): one wave a chunk, then the fold.
 extern "C" int ilm_attn_f32(void* out, void* ws, int nchunks, const void* q, const void* kc, const void* vc,
                             const void* block_tables, const void* seg, const void* pos, int T_, int nh, int nkv, int d,
-                            int page, int max_blocks, int q_stride, int out_stride, float scale, int window,
+                            int page, int max_blocks, int q_stride, int out_stride, float scale, int window, float softcap,
                             hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && nh > 0 && nkv > 0 && d > 0 && page > 0 && max_blocks > 0, "attn_f32: bad sizes");
     ILM_REQUIRE(nh % nkv == 0, "attn_f32: %d query heads do not divide into %d groups", nh, nkv);
@@ -273,7 +277,7 @@ extern "C" int ilm_attn_f32(void* out, void* ws, int nchunks, const void* q, con
     ILM_REQUIRE((long long)nkv * nsub <= 65535 && nh <= 65535, "attn_f32: too many heads");
     dim3 grid(T_, nkv * nsub, ws != nullptr ? nchunks : 1);
 #define FA_ARGS (float*)out, (float*)ws, (const float*)q, (const float*)kc, (const float*)vc, (const int*)block_tables, \
-                (const int*)seg, (const int*)pos, nh, nkv, nsub, page, max_blocks, q_stride, out_stride, scale, window
+                (const int*)seg, (const int*)pos, nh, nkv, nsub, page, max_blocks, q_stride, out_stride, scale, window, softcap
 #define FA_CASE(DT_)                                                                        \
     case DT_:                                                                               \
         if (ws != nullptr) attn_f32_kernel<DT_, true><<<grid, 64, 0, stream>>>(FA_ARGS);    \

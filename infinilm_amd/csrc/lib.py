@@ -41,15 +41,23 @@ _SIGNATURES = {
     "ilm_gemm_frag_tail": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _P],
     "ilm_gemm_f32_skinny": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
     "ilm_gemm_f32_tile": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
-    "ilm_attn_f32": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "ilm_attn_f32": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _F, _P],
     "ilm_gemm_basic": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
-    "ilm_attn_basic": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "ilm_attn_basic": [_P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _F, _P],
     "ilm_gemm_skinny": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ilm_attn_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
     "ilm_attn_mfma_static": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
     "ilm_attn_tile": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "ilm_argmax": [_P, _P, _I, _I, _I, _P],
     "ilm_sample": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
+    "ilm_unary": [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
+    "ilm_lin_prep": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "ilm_decay_scan": [_P, _I, _P, _P, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "ilm_group_norm_gate": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _I, _P],
+    "ilm_causal_conv": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P],
+    "ilm_ssm_steps": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "ilm_unit_qk_kvwrite": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P],
+    "ilm_weighted_sum": [_P, _P, _P, _L, _F, _F, _I, _I, _I, _P],
 }
 
 

@@ -1,0 +1,425 @@
+// Kernels of the mixers that carry a fixed-size state from token to token (linear attention with a decay,
+// selective state spaces) and of the small steps around them: activations, rotation by computed angles,
+// norms in groups with a gate, the short causal convolution, unit-norm queries and keys with a
+// position-dependent temperature, and a weighted sum of two branches.
+//
+// Everything that enters a recurrence is float: states, decays, step sizes, rotated queries and keys.  A
+// request's state passes from step to step through a row of a float pool, so cutting a prompt into portions
+// changes no bit: a token's result is a function of the state before it and of its own row.
+#include "common.h"
+
+__device__ __forceinline__ float ldf(const void* p, int dt, size_t i) {
+    return dt == ILM_DTYPE_F32 ? ((const float*)p)[i] : bf16_bits_to_f32(((const uint16_t*)p)[i]);
+}
+__device__ __forceinline__ void stf(void* p, int dt, size_t i, float v) {
+    if (dt == ILM_DTYPE_F32) ((float*)p)[i] = v;
+    else ((uint16_t*)p)[i] = __builtin_bit_cast(uint16_t, (__bf16)v);
+}
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+#define RC_ACT_NONE 0
+#define RC_ACT_SILU 1
+#define RC_ACT_SIGMOID 2
+#define RC_ACT_RELU2 3
+#define RC_ACT_GELU_TANH 4
+
+__device__ __forceinline__ float act_f(float x, int kind) {
+    switch (kind) {
+        case RC_ACT_SILU: return silu_f(x);
+        case RC_ACT_SIGMOID: return sigmoid_f(x);
+        case RC_ACT_RELU2: { const float r = fmaxf(x, 0.f); return r * r; }
+        case RC_ACT_GELU_TANH: return 0.5f * x * (1.0f + tanhf(0.7978845608028654f * (x + 0.044715f * x * x * x)));
+        default: return x;
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// out[t, j] = act(in[t, j]), rows of n elements with their own strides
+// ------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+unary_kernel(void* __restrict__ out, const void* __restrict__ in, int n, int out_stride, int in_stride, int kind,
+             int out_dt, int in_dt) {
+    const int t = blockIdx.y;
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if (j >= n) return;
+    stf(out, out_dt, (size_t)t * out_stride + j, act_f(ldf(in, in_dt, (size_t)t * in_stride + j), kind));
+}
+
+extern "C" int ilm_unary(void* out, const void* in, int T_, int n, int out_stride, int in_stride, int kind, int out_dt,
+                         int in_dt, hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && n > 0 && T_ <= 65535 * 32768, "unary: bad sizes T=%d n=%d", T_, n);
+    ILM_REQUIRE(kind >= 0 && kind <= RC_ACT_GELU_TANH, "unary: unknown activation %d", kind);
+    for (int t0 = 0; t0 < T_; t0 += 65535) {
+        const int rows = T_ - t0 < 65535 ? T_ - t0 : 65535;
+        const size_t eo = out_dt == ILM_DTYPE_F32 ? 4 : 2, ei = in_dt == ILM_DTYPE_F32 ? 4 : 2;
+        unary_kernel<<<dim3((n + 255) / 256, rows), 256, 0, stream>>>((char*)out + (size_t)t0 * out_stride * eo,
+                                                                      (const char*)in + (size_t)t0 * in_stride * ei, n,
+                                                                      out_stride, in_stride, kind, out_dt, in_dt);
+    }
+    ILM_LAUNCH_CHECK("unary");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Queries, keys and values of a linear-attention mixer made ready for the recurrence, as floats:
+// rows [q: heads*dk | k: heads*dk | v: heads*dv] of the fused projection -> the same layout in float, with an
+// activation on all three, then the first `rd` entries of each q and k head turned by the angle pos * freq[i]
+// (entry i paired with entry i + rd/2), then k times k_scale.  One block a token.
+// ------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+lin_prep_kernel(float* __restrict__ out, const void* __restrict__ in, const int* __restrict__ pos,
+                const float* __restrict__ freq, int heads, int dk, int dv, int rd, int in_stride, int act, float k_scale,
+                int in_dt) {
+    const int t = blockIdx.x;
+    const int nqk = heads * dk, n = 2 * nqk + heads * dv;
+    const size_t ib = (size_t)t * in_stride, ob = (size_t)t * n;
+    const int half = rd >> 1;
+    const float p = (float)pos[t];
+    // the turned pairs
+    const int pairs = 2 * heads * half;
+    for (int it = threadIdx.x; it < pairs; it += 256) {
+        const int hs = it / half, i = it % half;   // hs: q heads, then k heads
+        const size_t c = (size_t)hs * dk + i;
+        const float a = act_f(ldf(in, in_dt, ib + c), act), b = act_f(ldf(in, in_dt, ib + c + half), act);
+        const float ang = p * freq[i];
+        float sn, cs;
+        sincosf(ang, &sn, &cs);
+        const float sc = hs >= heads ? k_scale : 1.0f;
+        out[ob + c] = (a * cs - b * sn) * sc;
+        out[ob + c + half] = (b * cs + a * sn) * sc;
+    }
+    // what passes: the rest of the q and k heads, and v
+    const int rest = dk - rd;
+    for (int it = threadIdx.x; it < 2 * heads * rest; it += 256) {
+        const int hs = it / rest, i = rd + it % rest;
+        const size_t c = (size_t)hs * dk + i;
+        out[ob + c] = act_f(ldf(in, in_dt, ib + c), act) * (hs >= heads ? k_scale : 1.0f);
+    }
+    for (int j = 2 * nqk + threadIdx.x; j < n; j += 256) out[ob + j] = act_f(ldf(in, in_dt, ib + j), act);
+}
+
+extern "C" int ilm_lin_prep(void* out, const void* in, const void* pos, const void* freq, int T_, int heads, int dk, int dv,
+                            int rd, int in_stride, int act, float k_scale, int in_dt, hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && heads > 0 && dk > 0 && dv > 0, "lin_prep: bad sizes");
+    ILM_REQUIRE(rd >= 0 && rd <= dk && rd % 2 == 0, "lin_prep: %d turned entries do not fit a head of %d", rd, dk);
+    ILM_REQUIRE(rd == 0 || (freq != nullptr && pos != nullptr), "lin_prep: a rotation needs positions and frequencies");
+    ILM_REQUIRE(in_stride >= 2 * heads * dk + heads * dv, "lin_prep: rows of %d elements are too short", in_stride);
+    lin_prep_kernel<<<T_, 256, 0, stream>>>((float*)out, in, (const int*)pos, (const float*)freq, heads, dk, dv, rd, in_stride,
+                                            act, k_scale, in_dt);
+    ILM_LAUNCH_CHECK("lin_prep");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// The recurrence  S_t = a_t S_(t-1) + (b_t k_t) v_t^T,  o_t = S_t^T q_t + skip v_t  per (request, head), token by token.
+//
+// A block of 256 threads owns a head's state for VT = 256 / KP value columns: thread (kp, column) keeps the
+// SC_NK entries kp, kp + KP, kp + 2 KP, ... of the column's dk state entries in registers; a token's output is
+// the sum over the KP threads of a column (lanes of one wave, folded by shuffles).  The state pool holds a
+// head's state as [dv][dk] (the key index fastest), so a column's KP threads read consecutive floats.
+// a_t comes per head (decay_h) or per token and head (decay_t [T, heads]); b_t (kscale_t [T, heads]) and skip
+// (skip_h [heads]) may be absent.  Head h reads the q and k of group h / q_div.
+// Requests are the segments of the step: seg_offsets [R + 1] rows, state_in / state_out [R] pool rows.
+// ------------------------------------------------------------------------------------------
+#define SC_NK 8
+
+__global__ void __launch_bounds__(256)
+decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__ q, const float* __restrict__ k,
+                  int qk_stride, int q_div, const float* __restrict__ v, int v_stride,
+                  const float* __restrict__ decay_h, const float* __restrict__ decay_t,
+                  const float* __restrict__ kscale_t, const float* __restrict__ skip_h, float* __restrict__ pool,
+                  const int* __restrict__ state_in, const int* __restrict__ state_out,
+                  const int* __restrict__ seg_offsets, int heads, int dk, int dv, int KP) {
+    const int r = blockIdx.z, h = blockIdx.y;
+    const int t0 = seg_offsets[r], t1 = seg_offsets[r + 1];
+    if (t0 >= t1) return;
+    const int VT = 256 / KP;
+    const int kp = threadIdx.x % KP, vc = blockIdx.x * VT + threadIdx.x / KP;
+    const bool vok = vc < dv;
+    const size_t hs = (size_t)dk * dv;                       // floats of a head's state
+    const size_t row_in = ((size_t)state_in[r] * heads + h) * hs, row_out = ((size_t)state_out[r] * heads + h) * hs;
+    float S[SC_NK];
+#pragma unroll
+    for (int i = 0; i < SC_NK; ++i) {
+        const int ki = i * KP + kp;
+        S[i] = (vok && ki < dk) ? pool[row_in + (size_t)vc * dk + ki] : 0.f;
+    }
+    const int qoff = (h / q_div) * dk;
+    const float a_h = decay_h != nullptr ? decay_h[h] : 1.0f;
+    const float skip = skip_h != nullptr ? skip_h[h] : 0.f;
+    float qn[SC_NK], kn[SC_NK], vn, an, bn;
+#define SC_LOAD(T_)                                                                              \
+    {                                                                                            \
+        const float* qr = q + (size_t)(T_) * qk_stride + qoff;                                   \
+        const float* kr = k + (size_t)(T_) * qk_stride + qoff;                                   \
+        _Pragma("unroll") for (int i = 0; i < SC_NK; ++i) {                                      \
+            const int ki = i * KP + kp;                                                          \
+            qn[i] = ki < dk ? qr[ki] : 0.f;                                                      \
+            kn[i] = ki < dk ? kr[ki] : 0.f;                                                      \
+        }                                                                                        \
+        vn = vok ? v[(size_t)(T_) * v_stride + (size_t)h * dv + vc] : 0.f;                       \
+        an = decay_t != nullptr ? decay_t[(size_t)(T_) * heads + h] : a_h;                       \
+        bn = kscale_t != nullptr ? kscale_t[(size_t)(T_) * heads + h] : 1.0f;                    \
+    }
+    SC_LOAD(t0)
+    for (int t = t0; t < t1; ++t) {
+        float qc[SC_NK], kc[SC_NK];
+#pragma unroll
+        for (int i = 0; i < SC_NK; ++i) {
+            qc[i] = qn[i];
+            kc[i] = kn[i];
+        }
+        const float vcur = vn, a = an, bv = bn * vn;
+        if (t + 1 < t1) SC_LOAD(t + 1)
+        float acc = 0.f;
+#pragma unroll
+        for (int i = 0; i < SC_NK; ++i) {
+            S[i] = fmaf(a, S[i], kc[i] * bv);
+            acc = fmaf(S[i], qc[i], acc);
+        }
+        for (int off = 1; off < KP; off <<= 1) acc += __shfl_xor(acc, off, 64);
+        if (kp == 0 && vok) o[(size_t)t * o_stride + (size_t)h * dv + vc] = fmaf(skip, vcur, acc);
+    }
+#undef SC_LOAD
+    if (vok) {
+#pragma unroll
+        for (int i = 0; i < SC_NK; ++i) {
+            const int ki = i * KP + kp;
+            if (ki < dk) pool[row_out + (size_t)vc * dk + ki] = S[i];
+        }
+    }
+}
+
+extern "C" int ilm_decay_scan_max_dk() { return SC_NK * 64; }
+
+extern "C" int ilm_decay_scan(void* o, int o_stride, const void* q, const void* k, int qk_stride, int q_div, const void* v,
+                              int v_stride, const void* decay_h, const void* decay_t, const void* kscale_t,
+                              const void* skip_h, void* pool, const void* state_in, const void* state_out,
+                              const void* seg_offsets, int R, int heads, int dk, int dv, hipStream_t stream) {
+    ILM_REQUIRE(R > 0 && heads > 0 && dk > 0 && dv > 0, "decay_scan: bad sizes");
+    ILM_REQUIRE(dk <= SC_NK * 64, "decay_scan: %d state entries a column, at most %d", dk, SC_NK * 64);
+    ILM_REQUIRE(q_div > 0 && heads % q_div == 0, "decay_scan: %d heads do not divide into groups of %d", heads, q_div);
+    ILM_REQUIRE((decay_h != nullptr) != (decay_t != nullptr), "decay_scan: a decay per head or per token, one of them");
+    ILM_REQUIRE(R <= 65535 && heads <= 65535, "decay_scan: too many requests or heads");
+    int KP = 1;
+    while (KP * SC_NK < dk) KP <<= 1;
+    const int VT = 256 / KP;
+    dim3 grid((dv + VT - 1) / VT, heads, R);
+    decay_scan_kernel<<<grid, 256, 0, stream>>>((float*)o, o_stride, (const float*)q, (const float*)k, qk_stride, q_div,
+                                                (const float*)v, v_stride, (const float*)decay_h, (const float*)decay_t,
+                                                (const float*)kscale_t, (const float*)skip_h, (float*)pool,
+                                                (const int*)state_in, (const int*)state_out, (const int*)seg_offsets, heads,
+                                                dk, dv, KP);
+    ILM_LAUNCH_CHECK("decay_scan");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// RMS norm in groups with an optional gate, one wave a (row, group):
+//   y = x * act(gate)            (gate_before)
+//   y = y / sqrt(mean_group(y^2) + eps) * w       (w may be absent)
+//   y = y * act(gate)            (otherwise)
+// Sums run over a group in an order that depends on its size only.
+// ------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+group_norm_gate_kernel(void* __restrict__ out, const void* __restrict__ x, const void* __restrict__ gate,
+                       const void* __restrict__ w, int rows, int n, int groups, int x_stride, int gate_stride,
+                       int out_stride, float eps, int gate_act, int gate_before, int out_dt, int x_dt, int gate_dt, int w_dt) {
+    const int item = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (item >= rows * groups) return;
+    const int t = item / groups, g = item % groups, gs = n / groups;
+    const size_t xb = (size_t)t * x_stride + (size_t)g * gs, gb = (size_t)t * gate_stride + (size_t)g * gs;
+    const size_t ob = (size_t)t * out_stride + (size_t)g * gs;
+    const bool pre = gate != nullptr && gate_before;
+    float ss = 0.f;
+    for (int j = lane; j < gs; j += 64) {
+        float y = ldf(x, x_dt, xb + j);
+        if (pre) y *= act_f(ldf(gate, gate_dt, gb + j), gate_act);
+        ss = fmaf(y, y, ss);
+    }
+    ss = wave_sum(ss);
+    const float rstd = 1.0f / sqrtf(ss / (float)gs + eps);
+    for (int j = lane; j < gs; j += 64) {
+        float y = ldf(x, x_dt, xb + j);
+        if (pre) y *= act_f(ldf(gate, gate_dt, gb + j), gate_act);
+        y *= rstd;
+        if (w != nullptr) y *= ldf(w, w_dt, (size_t)g * gs + j);
+        if (gate != nullptr && !gate_before) y *= act_f(ldf(gate, gate_dt, gb + j), gate_act);
+        stf(out, out_dt, ob + j, y);
+    }
+}
+
+extern "C" int ilm_group_norm_gate(void* out, const void* x, const void* gate, const void* w, int rows, int n, int groups,
+                                   int x_stride, int gate_stride, int out_stride, float eps, int gate_act, int gate_before,
+                                   int out_dt, int x_dt, int gate_dt, int w_dt, hipStream_t stream) {
+    ILM_REQUIRE(rows > 0 && n > 0 && groups > 0 && n % groups == 0, "group_norm_gate: %d elements do not divide into %d groups", n, groups);
+    ILM_REQUIRE((long)rows * groups < (1L << 31) - 4, "group_norm_gate: too many rows");
+    const int blocks = (int)(((long)rows * groups + 3) / 4);
+    group_norm_gate_kernel<<<blocks, 256, 0, stream>>>(out, x, gate, w, rows, n, groups, x_stride, gate_stride, out_stride, eps,
+                                                      gate_act, gate_before, out_dt, x_dt, gate_dt, w_dt);
+    ILM_LAUNCH_CHECK("group_norm_gate");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Short causal convolution over the tokens of each request, per channel, with bias and activation:
+//   y[t, c] = act(b[c] + sum_i w[c, i] * x[t - (taps - 1) + i, c]),   the last tap is the token's own input.
+// Inputs before a request's first token of this step come from its state row (the last taps - 1 inputs of the
+// steps before, oldest first; zeros for a new request); the row is then written anew.  One thread a (request,
+// channel) walks the request's tokens with the window in registers, so a state entry has one reader and writer.
+// ------------------------------------------------------------------------------------------
+#define CV_MAX_TAPS 8
+
+__global__ void __launch_bounds__(256)
+causal_conv_kernel(float* __restrict__ y, const void* __restrict__ x, const void* __restrict__ w, const void* __restrict__ b,
+                   float* __restrict__ pool, const int* __restrict__ state_in, const int* __restrict__ state_out,
+                   const int* __restrict__ seg_offsets, int C, int taps, int x_stride, int y_stride, int act, int x_dt, int w_dt) {
+    const int r = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int t0 = seg_offsets[r], t1 = seg_offsets[r + 1];
+    if (t0 >= t1) return;
+    float win[CV_MAX_TAPS], wt[CV_MAX_TAPS];
+    const size_t sin = (size_t)state_in[r] * (taps - 1) * C, sout = (size_t)state_out[r] * (taps - 1) * C;
+#pragma unroll
+    for (int i = 0; i < CV_MAX_TAPS; ++i) {
+        wt[i] = i < taps ? ldf(w, w_dt, (size_t)c * taps + i) : 0.f;
+        win[i] = i < taps - 1 ? pool[sin + (size_t)i * C + c] : 0.f;
+    }
+    const float bias = b != nullptr ? ldf(b, w_dt, c) : 0.f;
+    const float w_last = ldf(w, w_dt, (size_t)c * taps + taps - 1);   // the token's own tap
+    for (int t = t0; t < t1; ++t) {
+        const float xv = ldf(x, x_dt, (size_t)t * x_stride + c);
+        float s = bias;
+#pragma unroll
+        for (int i = 0; i < CV_MAX_TAPS; ++i) {
+            if (i < taps - 1) s = fmaf(wt[i], win[i], s);
+        }
+        s = fmaf(w_last, xv, s);
+        y[(size_t)t * y_stride + c] = act_f(s, act);
+#pragma unroll
+        for (int i = 0; i < CV_MAX_TAPS - 1; ++i) win[i] = (i + 1 < taps - 1) ? win[i + 1] : (i == taps - 2 ? xv : win[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < CV_MAX_TAPS; ++i)
+        if (i < taps - 1) pool[sout + (size_t)i * C + c] = win[i];
+}
+
+extern "C" int ilm_causal_conv_max_taps() { return CV_MAX_TAPS; }
+
+extern "C" int ilm_causal_conv(void* y, const void* x, const void* w, const void* b, void* pool, const void* state_in,
+                               const void* state_out, const void* seg_offsets, int R, int C, int taps, int x_stride,
+                               int y_stride, int act, int x_dt, int w_dt, hipStream_t stream) {
+    ILM_REQUIRE(R > 0 && C > 0 && R <= 65535, "causal_conv: bad sizes");
+    ILM_REQUIRE(taps >= 1 && taps <= CV_MAX_TAPS, "causal_conv: %d taps, at most %d", taps, CV_MAX_TAPS);
+    causal_conv_kernel<<<dim3((C + 255) / 256, R), 256, 0, stream>>>((float*)y, x, w, b, (float*)pool, (const int*)state_in,
+                                                                     (const int*)state_out, (const int*)seg_offsets, C, taps,
+                                                                     x_stride, y_stride, act, x_dt, w_dt);
+    ILM_LAUNCH_CHECK("causal_conv");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Step sizes and decays of a selective state space: dt = softplus(raw + bias[h]), decay = exp(-exp(A_log[h]) dt).
+// ------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+ssm_steps_kernel(float* __restrict__ dt, float* __restrict__ decay, const void* __restrict__ raw,
+                 const float* __restrict__ bias, const float* __restrict__ a_log, int T_, int heads, int raw_stride, int raw_dt) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= T_ * heads) return;
+    const int t = i / heads, h = i % heads;
+    const float z = ldf(raw, raw_dt, (size_t)t * raw_stride + h) + bias[h];
+    const float d = z > 20.0f ? z : log1pf(expf(z));
+    dt[i] = d;
+    decay[i] = expf(-expf(a_log[h]) * d);
+}
+
+extern "C" int ilm_ssm_steps(void* dt, void* decay, const void* raw, const void* bias, const void* a_log, int T_, int heads,
+                             int raw_stride, int raw_dt, hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && heads > 0, "ssm_steps: bad sizes");
+    ssm_steps_kernel<<<(T_ * heads + 255) / 256, 256, 0, stream>>>((float*)dt, (float*)decay, raw, (const float*)bias,
+                                                                   (const float*)a_log, T_, heads, raw_stride, raw_dt);
+    ILM_LAUNCH_CHECK("ssm_steps");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// Queries and keys of unit root mean square with a temperature on the queries, inside the fused projection
+// rows [T, (nh + 2 nkv) d], and k, v into the paged cache (keys [pages, nkv, page, d], values [pages, nkv, d, page]).
+// A head has `dn` entries that count (the rest up to d are zeros that only fill the head up):
+//   q <- q / sqrt(sum(q^2) / dn + eps) * (1 + coef * ln(floor((pos + 1) / every) + 1)),  k <- k / sqrt(sum(k^2) / dn + eps).
+// normed == 0: no division.  every <= 0: no temperature.  One wave a (token, head).
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(64)
+unit_qk_kvwrite_kernel(T* __restrict__ qkv, const int* __restrict__ pos, T* __restrict__ kc, T* __restrict__ vc,
+                       const int* __restrict__ slots, int nh, int nkv, int d, int dn, int row_stride, int page, int normed,
+                       float eps, float coef, int every) {
+    const int t = blockIdx.x, hs = blockIdx.y, lane = threadIdx.x;
+    T* p = qkv + (size_t)t * row_stride + (size_t)hs * d;
+    const int slot = slots != nullptr ? slots[t] : -1;
+    if (hs >= nh + nkv) {
+        if (slot >= 0) {
+            T* vdst = vc + ((size_t)(slot / page) * nkv + (hs - nh - nkv)) * d * page + (slot % page);
+            for (int i = lane; i < d; i += 64) vdst[(size_t)i * page] = p[i];
+        }
+        return;
+    }
+    const bool is_k = hs >= nh;
+    float f = 1.0f;
+    if (normed) {
+        float ss = 0.f;
+        for (int i = lane; i < d; i += 64) {
+            const float x = to_f32(p[i]);
+            ss = fmaf(x, x, ss);
+        }
+        f = 1.0f / sqrtf(wave_sum(ss) / (float)dn + eps);
+    }
+    if (!is_k && every > 0) f *= 1.0f + coef * logf((float)((pos[t] + 1) / every) + 1.0f);
+    T* dst = (is_k && slot >= 0) ? kc + (((size_t)(slot / page) * nkv + (hs - nh)) * page + (slot % page)) * d : nullptr;
+    for (int i = lane; i < d; i += 64) {
+        const T y = from_f32<T>(to_f32(p[i]) * f);
+        p[i] = y;
+        if (dst != nullptr) dst[i] = y;
+    }
+}
+
+extern "C" int ilm_unit_qk_kvwrite(void* qkv, const void* pos, void* kc, void* vc, const void* slots, int T_, int nh, int nkv,
+                                   int d, int dn, int row_stride, int page, int normed, float eps, float coef, int every,
+                                   int dtype, hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && nh > 0 && nkv > 0 && d > 0 && dn > 0 && dn <= d, "unit_qk_kvwrite: bad sizes");
+    ILM_REQUIRE(nh + 2 * nkv <= 65535, "unit_qk_kvwrite: too many heads");
+    ILM_REQUIRE(slots == nullptr || (kc != nullptr && vc != nullptr && page > 0), "unit_qk_kvwrite: slots without a cache");
+    dim3 grid(T_, nh + 2 * nkv);
+    if (dtype == ILM_DTYPE_F32)
+        unit_qk_kvwrite_kernel<float><<<grid, 64, 0, stream>>>((float*)qkv, (const int*)pos, (float*)kc, (float*)vc,
+                                                              (const int*)slots, nh, nkv, d, dn, row_stride, page, normed, eps,
+                                                              coef, every);
+    else if (dtype == ILM_DTYPE_BF16)
+        unit_qk_kvwrite_kernel<bf16><<<grid, 64, 0, stream>>>((bf16*)qkv, (const int*)pos, (bf16*)kc, (bf16*)vc,
+                                                             (const int*)slots, nh, nkv, d, dn, row_stride, page, normed, eps,
+                                                             coef, every);
+    else
+        ILM_REQUIRE(false, "unit_qk_kvwrite: unknown dtype %d", dtype);
+    ILM_LAUNCH_CHECK("unit_qk_kvwrite");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// out = a x + b y, element by element (the branches of a mixer that runs two side by side)
+// ------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+weighted_sum_kernel(void* __restrict__ out, const void* __restrict__ x, const void* __restrict__ y, long n, float a, float b,
+                    int out_dt, int x_dt, int y_dt) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n) return;
+    stf(out, out_dt, i, fmaf(a, ldf(x, x_dt, i), b * ldf(y, y_dt, i)));
+}
+
+extern "C" int ilm_weighted_sum(void* out, const void* x, const void* y, long n, float a, float b, int out_dt, int x_dt,
+                                int y_dt, hipStream_t stream) {
+    ILM_REQUIRE(n > 0 && (n + 255) / 256 < (1L << 31), "weighted_sum: bad size");
+    weighted_sum_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(out, x, y, n, a, b, out_dt, x_dt, y_dt);
+    ILM_LAUNCH_CHECK("weighted_sum");
+    return 0;
+}

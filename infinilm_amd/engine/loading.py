@@ -95,7 +95,8 @@ def pages_that_fit(model: CausalLM, page_size: int, memory_fraction: float = 0.9
     from ..cache.needs import PagedKV
     reserve_bytes += fragment_copy_bytes(model)
     elem = torch.empty((), dtype=model.dtype).element_size()
-    per_page = sum(2 * n.num_kv_heads * n.head_dim * page_size * elem for n in model.cache_needs if isinstance(n, PagedKV))
+    flat = [m for n in model.cache_needs for m in (n if isinstance(n, (tuple, list)) else (n,))]
+    per_page = sum(2 * n.num_kv_heads * n.head_dim * page_size * elem for n in flat if isinstance(n, PagedKV))
     if per_page == 0:
         return 1
     free, _ = torch.cuda.mem_get_info(model.device)

@@ -16,6 +16,7 @@ import torch
 from .. import kernels
 from ..config.spec import ModelSpec, PartSpec
 from ..parts import BuildContext, Param, ResidualStream, build_block
+from ..parts.base import join_name
 from ..parts.registry import build_embedding, build_head, build_norm
 
 
@@ -32,6 +33,8 @@ class CausalLM:
         self.final_norm = build_norm(spec.final_norm, ctx)
         self.output_head = build_head(PartSpec(spec.head.kind, dict(spec.head.params, vocab_size=spec.vocab_size,
                                                                     hidden_size=spec.hidden_size, scale=spec.head.scale)), ctx)
+        if spec.head.always_tied:
+            self.output_head.tie(self.embedding.table)
         # cache entry -> what its writer's mixer needs
         self.cache_needs: List = [None] * spec.num_cache_entries()
         for run in spec.order:
@@ -62,13 +65,14 @@ class CausalLM:
     def named_parameters(self) -> Dict[str, Param]:
         out: Dict[str, Param] = {}
         for name, p in self.embedding.named_parameters().items():
-            out[f"{self.spec.embed_name}.{name}"] = p
+            out[join_name(self.spec.embed_name, name)] = p
         for b in self.blocks:
             out.update(b.named_parameters())
         for name, p in self.final_norm.named_parameters().items():
-            out[f"{self.spec.final_norm_name}.{name}"] = p
-        for name, p in self.output_head.named_parameters().items():
-            out[f"{self.spec.head.name}.{name}"] = p
+            out[join_name(self.spec.final_norm_name, name)] = p
+        if not self.spec.head.always_tied:
+            for name, p in self.output_head.named_parameters().items():
+                out[join_name(self.spec.head.name, name)] = p
         return out
 
     def tie_head_to_embedding(self) -> None:

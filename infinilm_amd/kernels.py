@@ -671,8 +671,10 @@ def attention_chunks(max_total_len: int, page: int, pairs: int, device) -> tuple
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                     seg_of_token: torch.Tensor, positions: torch.Tensor, nh: int, nkv: int, d: int,
                     scale: float, window: int = 0, max_total_len: Optional[int] = None,
-                    tiles: Optional[torch.Tensor] = None, single_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    tiles: Optional[torch.Tensor] = None, single_rows: Optional[torch.Tensor] = None,
+                    softcap: float = 0.0) -> torch.Tensor:
     """Attention of every token over its request's cached keys up to its own position.
+    `softcap` > 0: scaled scores pass through softcap * tanh(score / softcap) before the softmax.
 
     q: rows of T tokens in which head h lies at [h*d, (h+1)*d) (a view into the fused projection is
     fine); caches as the cache manager lays them out; block_tables [R, max_blocks]; `max_total_len`: an
@@ -694,7 +696,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         raise KernelError("per-token metadata does not match the number of tokens")
     out = torch.empty((T, nh * d), dtype=q.dtype, device=q.device)
     if (q.dtype == BF16 and not FORCE_BASIC and d % 16 == 0 and d <= 128 and page % 16 == 0 and q.stride(0) % 8 == 0
-            and max_total_len is not None):
+            and max_total_len is not None and not softcap > 0.0):
         n_single = T
         rows = None
         if tiles is not None and tiles.numel() > 0:
@@ -732,7 +734,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             ws = torch.empty((T * nh * nchunks * (d + 4),), dtype=F32, device=q.device)
         _run("ilm_attn_f32", out.data_ptr(), _ptr(ws), nchunks, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
              block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d, page,
-             block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window), _stream())
+             block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window), float(softcap), _stream())
         return out
     # The plain kernel.  Few tokens over long contexts (decoding): one wave a chunk of keys and a fold of the
     # partial results, instead of one wave a head; the bits are the same (see attn_basic.hip).
@@ -742,7 +744,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         ws = torch.empty((T * nh * nchunks * (d + 2),), dtype=F32, device=q.device)
     _run("ilm_attn_basic", out.data_ptr(), _ptr(ws), nchunks, q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
          block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), T, nh, nkv, d, page, block_tables.shape[1],
-         q.stride(0), out.stride(0), float(scale), int(window), _dt(q), _stream())
+         q.stride(0), out.stride(0), float(scale), int(window), _dt(q), float(softcap), _stream())
     return out
 
 
@@ -1009,3 +1011,192 @@ def gemm_frag_tail(x: FragRows, fw: FragWeight, bias: Optional[torch.Tensor], al
          fw.data.data_ptr(), _ptr(bias), norm_w.data_ptr(), 1 if norm_w.dtype == F32 else 0, float(alpha), M, N, fw.K,
          FRAG_TILES, _stream())
     return xw, ss
+
+
+# ---- mixers with a fixed-size state, and the small steps around them -------------------------------------------------
+ACTIVATIONS = {"none": 0, "silu": 1, "sigmoid": 2, "relu2": 3, "gelu_tanh": 4}
+SCAN_MAX_KEY_DIM = 512      # most state entries a value column of the recurrence (ilm_decay_scan_max_dk())
+CONV_MAX_TAPS = 8           # most taps of the short convolution (ilm_causal_conv_max_taps())
+
+
+def _act(kind: str) -> int:
+    try:
+        return ACTIVATIONS[kind]
+    except KeyError:
+        raise KernelError(f"unknown activation {kind!r}; known: {sorted(ACTIVATIONS)}") from None
+
+
+def _rows(x: torch.Tensor, name: str) -> None:
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise KernelError(f"{name} must be a matrix with dense rows")
+
+
+def activation(x: torch.Tensor, kind: str, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """act(x) element by element; x [T, n] with dense rows (a view into wider rows is fine)."""
+    _dev(x)
+    _rows(x, "x")
+    T, n = x.shape
+    out = torch.empty((T, n), dtype=out_dtype or x.dtype, device=x.device)
+    _run("ilm_unary", out.data_ptr(), x.data_ptr(), T, n, out.stride(0), x.stride(0), _act(kind), _dt(out), _dt(x), _stream())
+    return out
+
+
+def linear_attention_inputs(qkv: torch.Tensor, positions: Optional[torch.Tensor], freq: Optional[torch.Tensor], heads: int,
+                            dk: int, dv: int, rotary_dims: int, act: str, k_scale: float) -> torch.Tensor:
+    """float32 rows [q: heads*dk | k: heads*dk | v: heads*dv] from the fused projection's rows of the same layout:
+    an activation on all, q and k turned by position * freq[i] on their first `rotary_dims` entries (entry i paired
+    with entry i + rotary_dims/2), k times `k_scale`."""
+    _dev(qkv, positions, freq)
+    _rows(qkv, "qkv")
+    T = qkv.shape[0]
+    n = heads * (2 * dk + dv)
+    if qkv.shape[1] < n:
+        raise KernelError(f"rows of {qkv.shape[1]} do not hold q, k and v of {heads} heads of {dk} / {dv}")
+    if rotary_dims:
+        if positions is None or freq is None:
+            raise KernelError("a rotation needs positions and frequencies")
+        _i32(positions, "positions")
+        if positions.numel() != T or freq.dtype != F32 or freq.numel() != rotary_dims // 2 or not freq.is_contiguous():
+            raise KernelError(f"frequencies must be float32 [{rotary_dims // 2}] and positions one a token")
+    out = torch.empty((T, n), dtype=F32, device=qkv.device)
+    _run("ilm_lin_prep", out.data_ptr(), qkv.data_ptr(), _ptr(positions), _ptr(freq), T, heads, dk, dv, int(rotary_dims),
+         qkv.stride(0), _act(act), float(k_scale), _dt(qkv), _stream())
+    return out
+
+
+def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, dk: int, dv: int, groups: int,
+               pool: torch.Tensor, state_in: torch.Tensor, state_out: torch.Tensor, seg_offsets: torch.Tensor, segments: int,
+               decay_h: Optional[torch.Tensor] = None, decay_t: Optional[torch.Tensor] = None,
+               kscale_t: Optional[torch.Tensor] = None, skip_h: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """S_t = a_t S_(t-1) + (b_t k_t) v_t^T, o_t = S_t^T q_t + skip_h v_t for every head of every segment, token by token,
+    all in float32.  q, k: [T, groups*dk] (views with one row stride; head h reads group h // (heads/groups)), v [T, heads*dv];
+    a per head (`decay_h` [heads]) or per token (`decay_t` [T, heads]); b `kscale_t` [T, heads] or absent.  `pool`
+    [rows, heads, dv, dk] holds the states: segment r starts from row state_in[r] and leaves its state in row state_out[r].
+    Returns o [T, heads*dv]."""
+    _dev(q, k, v, pool, state_in, state_out, seg_offsets, decay_h, decay_t, kscale_t, skip_h)
+    for t, nm in ((q, "q"), (k, "k"), (v, "v")):
+        _rows(t, nm)
+        if t.dtype != F32:
+            raise KernelError(f"{nm} of the recurrence must be float32")
+    T = v.shape[0]
+    if q.shape != (T, groups * dk) or k.shape != (T, groups * dk) or v.shape != (T, heads * dv) or q.stride(0) != k.stride(0):
+        raise KernelError(f"recurrence operands {tuple(q.shape)}, {tuple(k.shape)}, {tuple(v.shape)} do not fit {heads} heads "
+                          f"in {groups} groups of {dk} / {dv}")
+    if groups <= 0 or heads % groups or dk > SCAN_MAX_KEY_DIM:
+        raise KernelError(f"{heads} heads in {groups} groups, key size {dk} (at most {SCAN_MAX_KEY_DIM})")
+    if pool.dtype != F32 or not pool.is_contiguous() or tuple(pool.shape[1:]) != (heads, dv, dk):
+        raise KernelError(f"the state pool must be float32 [rows, {heads}, {dv}, {dk}], got {tuple(pool.shape)}")
+    for t, nm in ((state_in, "state_in"), (state_out, "state_out"), (seg_offsets, "seg_offsets")):
+        _i32(t, nm)
+    if state_in.numel() < segments or state_out.numel() < segments or seg_offsets.numel() < segments + 1:
+        raise KernelError("state rows and offsets must cover every segment")
+    for t, shape, nm in ((decay_h, (heads,), "decay_h"), (decay_t, (T, heads), "decay_t"), (kscale_t, (T, heads), "kscale_t"),
+                         (skip_h, (heads,), "skip_h")):
+        if t is not None and (t.dtype != F32 or tuple(t.shape) != shape or not t.is_contiguous()):
+            raise KernelError(f"{nm} must be contiguous float32 {shape}")
+    if (decay_h is None) == (decay_t is None):
+        raise KernelError("the recurrence takes a decay per head or per token, one of them")
+    o = torch.empty((T, heads * dv), dtype=F32, device=v.device)
+    _run("ilm_decay_scan", o.data_ptr(), o.stride(0), q.data_ptr(), k.data_ptr(), q.stride(0), heads // groups, v.data_ptr(),
+         v.stride(0), _ptr(decay_h), _ptr(decay_t), _ptr(kscale_t), _ptr(skip_h), pool.data_ptr(), state_in.data_ptr(),
+         state_out.data_ptr(), seg_offsets.data_ptr(), int(segments), heads, dk, dv, _stream())
+    return o
+
+
+def group_norm_gate(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, groups: int = 1,
+                    gate: Optional[torch.Tensor] = None, gate_act: str = "none", gate_before: bool = False,
+                    out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """RMS norm of every row in `groups` equal parts (each by its own root mean square, eps inside the root), times
+    `weight` [n] if given; `gate` [T, n]: times act(gate), before the norm or after it.  Sums in float32."""
+    _dev(x, weight, gate)
+    _rows(x, "x")
+    T, n = x.shape
+    if groups <= 0 or n % groups:
+        raise KernelError(f"rows of {n} do not divide into {groups} groups")
+    if weight is not None and (weight.shape != (n,) or not weight.is_contiguous()):
+        raise KernelError(f"norm weight has shape {tuple(weight.shape)}, expected ({n},)")
+    if gate is not None:
+        _rows(gate, "gate")
+        if gate.shape != (T, n):
+            raise KernelError(f"gate {tuple(gate.shape)} does not match {tuple(x.shape)}")
+    out = torch.empty((T, n), dtype=out_dtype or x.dtype, device=x.device)
+    _run("ilm_group_norm_gate", out.data_ptr(), x.data_ptr(), _ptr(gate), _ptr(weight), T, n, int(groups), x.stride(0),
+         gate.stride(0) if gate is not None else 0, out.stride(0), float(eps), _act(gate_act), int(bool(gate_before)),
+         _dt(out), _dt(x), _dt(gate) if gate is not None else 0, _dt(weight) if weight is not None else 0, _stream())
+    return out
+
+
+def causal_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], pool: torch.Tensor,
+                state_in: torch.Tensor, state_out: torch.Tensor, seg_offsets: torch.Tensor, segments: int,
+                act: str = "silu") -> torch.Tensor:
+    """y[t, c] = act(bias[c] + sum_i weight[c, i] x[t - taps + 1 + i, c]) over the tokens of each segment; what lies
+    before a segment's first row comes from its row of `pool` [rows, taps - 1, channels] (float32, oldest first), which
+    is then written anew (row state_out[r]).  float32 result [T, channels]."""
+    _dev(x, weight, bias, pool, state_in, state_out, seg_offsets)
+    _rows(x, "x")
+    T, C = x.shape
+    if weight.dim() != 2 or weight.shape[0] != C or not weight.is_contiguous() or not 1 <= weight.shape[1] <= CONV_MAX_TAPS:
+        raise KernelError(f"convolution weight {tuple(weight.shape)} must be [{C}, taps <= {CONV_MAX_TAPS}]")
+    taps = weight.shape[1]
+    if bias is not None and (bias.shape != (C,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
+        raise KernelError("convolution bias does not fit its weight")
+    if pool.dtype != F32 or not pool.is_contiguous() or tuple(pool.shape[1:]) != (max(taps - 1, 0), C):
+        raise KernelError(f"the convolution's state pool must be float32 [rows, {taps - 1}, {C}], got {tuple(pool.shape)}")
+    for t, nm in ((state_in, "state_in"), (state_out, "state_out"), (seg_offsets, "seg_offsets")):
+        _i32(t, nm)
+    if state_in.numel() < segments or state_out.numel() < segments or seg_offsets.numel() < segments + 1:
+        raise KernelError("state rows and offsets must cover every segment")
+    y = torch.empty((T, C), dtype=F32, device=x.device)
+    _run("ilm_causal_conv", y.data_ptr(), x.data_ptr(), weight.data_ptr(), _ptr(bias), pool.data_ptr(), state_in.data_ptr(),
+         state_out.data_ptr(), seg_offsets.data_ptr(), int(segments), C, taps, x.stride(0), y.stride(0), _act(act), _dt(x),
+         _dt(weight), _stream())
+    return y
+
+
+def ssm_steps(raw: torch.Tensor, bias: torch.Tensor, a_log: torch.Tensor):
+    """(dt, decay), float32 [T, heads]: dt = softplus(raw + bias), decay = exp(-exp(a_log) dt)."""
+    _dev(raw, bias, a_log)
+    _rows(raw, "raw step sizes")
+    T, H = raw.shape
+    for t, nm in ((bias, "bias"), (a_log, "a_log")):
+        if t.dtype != F32 or t.shape != (H,) or not t.is_contiguous():
+            raise KernelError(f"{nm} must be contiguous float32 [{H}]")
+    dt = torch.empty((T, H), dtype=F32, device=raw.device)
+    decay = torch.empty((T, H), dtype=F32, device=raw.device)
+    _run("ilm_ssm_steps", dt.data_ptr(), decay.data_ptr(), raw.data_ptr(), bias.data_ptr(), a_log.data_ptr(), T, H,
+         raw.stride(0), _dt(raw), _stream())
+    return dt, decay
+
+
+def unit_qk_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, k_cache: Optional[torch.Tensor],
+                    v_cache: Optional[torch.Tensor], slots: Optional[torch.Tensor], nh: int, nkv: int, d: int, dn: int,
+                    normed: bool, eps: float, coef: float, every: int) -> None:
+    """Inside the fused rows [T, (nh + 2 nkv) d]: q and k heads divided by their root mean square over their `dn` entries
+    that count (if `normed`), q times 1 + coef * ln(floor((position + 1) / every) + 1) (if every > 0); then k and v go
+    to the paged cache at `slots` (None: no write)."""
+    _dev(qkv, positions, k_cache, v_cache, slots)
+    _rows(qkv, "qkv")
+    _i32(positions, "positions")
+    T = qkv.shape[0]
+    if qkv.shape[1] < (nh + 2 * nkv) * d or positions.numel() != T or not 0 < dn <= d:
+        raise KernelError("fused rows do not hold the heads, or positions do not match the tokens")
+    page = 0
+    if slots is not None:
+        _i32(slots, "slots")
+        if k_cache is None or v_cache is None or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
+            raise KernelError("cache tensors missing or of another dtype than the activations")
+        page = _check_cache(k_cache, v_cache, nkv, d)
+    _run("ilm_unit_qk_kvwrite", qkv.data_ptr(), positions.data_ptr(), _ptr(k_cache) if slots is not None else None,
+         _ptr(v_cache) if slots is not None else None, _ptr(slots), T, nh, nkv, d, int(dn), qkv.stride(0), page,
+         int(bool(normed)), float(eps), float(coef), int(every), _dt(qkv), _stream())
+
+
+def weighted_sum(x: torch.Tensor, y: torch.Tensor, a: float, b: float, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """a x + b y, element by element."""
+    _dev(x, y)
+    if x.shape != y.shape or not x.is_contiguous() or not y.is_contiguous():
+        raise KernelError("weighted_sum takes two contiguous tensors of one shape")
+    out = torch.empty(x.shape, dtype=out_dtype or x.dtype, device=x.device)
+    _run("ilm_weighted_sum", out.data_ptr(), x.data_ptr(), y.data_ptr(), x.numel(), float(a), float(b), _dt(out), _dt(x),
+         _dt(y), _stream())
+    return out

@@ -1,4 +1,5 @@
-from . import attention, block, ends, mlp, norm, rotary  # noqa: F401  (register the built-in kinds)
+from . import (attention, block, ends, linear_attention, mlp, norm, parallel, rotary, state_space,  # noqa: F401
+               temperature)   # (register the built-in kinds)
 from .base import (BuildContext, FeedForward, Mixer, Norm, Param, Part, PositionEncoding, ResidualStream)
 from .block import build_block
 from .ends import Embedding, OutputHead

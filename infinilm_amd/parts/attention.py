@@ -8,7 +8,7 @@ prompts and single decoded tokens: a token at position p sees its request's keys
 """
 from __future__ import annotations
 
-from typing import Dict
+from typing import Dict, Optional, Sequence
 
 import torch
 
@@ -22,16 +22,37 @@ from .registry import build_position_encoding, register_mixer
 
 @register_mixer("gqa_attention")
 class GQAttention(Mixer):
+    """`value_dim`: the size of a value head where it differs from the query and key heads'; `softcap` > 0: scaled
+    scores pass through softcap * tanh(score / softcap); `names`, `suffix`: the projections' tensor names in a
+    checkpoint; `whole_output`: the result comes as one [T, hidden] tensor in the activations' dtype (never as float32
+    parts still to be summed), for an arrangement that does more with it than add it to the residual stream.
+
+    The cache and the attention kernels know one head size: query/key heads and value heads of different sizes (or
+    of a size that is no multiple of 16) are filled up with zeros to the next multiple of 16 that holds both, in the
+    projections' weights: zero entries add nothing to a score, and the output entries they make meet zero columns
+    of the output projection."""
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, qkv_bias: bool,
-                 out_bias: bool, scale: float, window: int, position: PartSpec, ctx: BuildContext):
+                 out_bias: bool, scale: float, window: int, position: PartSpec, ctx: BuildContext,
+                 value_dim: Optional[int] = None, softcap: float = 0.0,
+                 names: Sequence[str] = ("q_proj", "k_proj", "v_proj", "o_proj"), suffix: str = "weight",
+                 whole_output: bool = False):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads do not divide into {num_kv_heads} groups")
-        self.nh, self.nkv, self.d = int(num_heads), int(num_kv_heads), int(head_dim)
+        self.nh, self.nkv = int(num_heads), int(num_kv_heads)
+        self.dn = int(head_dim)                                       # entries of a query or key head that count
+        self.dv = int(value_dim) if value_dim is not None else self.dn
+        self.d = self.dn if self.dv == self.dn else -(-max(self.dn, self.dv) // 16) * 16   # the head size that runs
         self.scale = float(scale)
+        self.softcap = float(softcap)
         self.window = int(window)
-        self.qkv = FusedLinear(hidden_size, [self.nh * self.d, self.nkv * self.d, self.nkv * self.d],
-                               ["q_proj", "k_proj", "v_proj"], qkv_bias, ctx)
-        self.o_proj = Linear(self.nh * self.d, hidden_size, "o_proj", out_bias, ctx)
+        self.whole_output = bool(whole_output)
+        qn, kn, vn, on = names
+        self.qkv = FusedLinear(hidden_size, [self.nh * self.d, self.nkv * self.d, self.nkv * self.d], [qn, kn, vn],
+                               qkv_bias, ctx, suffix=suffix,
+                               out_heads=[(self.nh, self.dn, self.d), (self.nkv, self.dn, self.d), (self.nkv, self.dv, self.d)])
+        self.o_proj = Linear(self.nh * self.d, hidden_size, on, out_bias, ctx, suffix=suffix,
+                             in_heads=(self.nh, self.dv, self.d))
         self.position = build_position_encoding(position, ctx)
         if getattr(self.position, "head_dim", self.d) not in (0, self.d):
             raise ValueError(f"the position encoding is made for heads of {self.position.head_dim}, the mixer's have {self.d}")
@@ -66,9 +87,9 @@ class GQAttention(Mixer):
                 batch.taps.setdefault("qkv_rotated", []).append(qkv.clone())
         o = kernels.paged_attention(qkv, cache_view.k, cache_view.v, cache_view.block_tables, batch.seg_of_token,
                                     batch.positions, self.nh, self.nkv, self.d, self.scale, self.window,
-                                    batch.max_total_len, batch.att_tiles, batch.att_single_rows)
+                                    batch.max_total_len, batch.att_tiles, batch.att_single_rows, softcap=self.softcap)
         if tail is not None:   # the output projection adds into the residual stream itself, where its kernel can
             deferred = self.o_proj.forward_tail(o, tail)
             if deferred is not None:
                 return deferred
-        return self.o_proj.forward(o, allow_parts=True)
+        return self.o_proj.forward(o, allow_parts=not self.whole_output)

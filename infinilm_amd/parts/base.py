@@ -37,15 +37,31 @@ class Param:
     drawn around it."""
 
     def __init__(self, tensor: torch.Tensor, keep_f32: bool = False,
-                 replace: Optional[Callable[[torch.Tensor], None]] = None, neutral: float = 0.0):
+                 replace: Optional[Callable[[torch.Tensor], None]] = None, neutral: float = 0.0,
+                 shape: Optional[tuple] = None):
         self.tensor = tensor
         self.keep_f32 = keep_f32 and replace is not None
         self._replace = replace
         self.neutral = float(neutral)
+        # the tensor's shape in a checkpoint; `tensor` may be a strided view of the same elements in another shape
+        # (heads filled up with zeros to a size the kernels take)
+        self.shape = tuple(shape) if shape is not None else tuple(tensor.shape)
+        if shape is not None and self.keep_f32:
+            raise ValueError("a parameter stored through a view cannot be replaced")
 
     def replace(self, t: torch.Tensor) -> None:
         self._replace(t)
         self.tensor = t
+
+    def store(self, t: torch.Tensor) -> None:
+        """Copies a checkpoint's tensor (of shape `shape`) into the parameter."""
+        self.tensor.copy_(t.to(self.tensor.dtype).reshape(self.tensor.shape))
+
+
+def join_name(*pieces: str) -> str:
+    """Pieces of a tensor's name joined by dots; empty pieces are left out (a part whose one tensor carries the
+    part's own name gives it the name "")."""
+    return ".".join(p for p in pieces if p)
 
 
 class Part:

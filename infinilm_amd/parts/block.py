@@ -9,7 +9,7 @@ from __future__ import annotations
 from typing import Dict
 
 from ..config.spec import LayerSpec
-from .base import BuildContext, DeferredNorm, Param, ResidualStream
+from .base import BuildContext, DeferredNorm, Param, ResidualStream, join_name
 from .registry import ARRANGEMENTS, build_feed_forward, build_mixer, build_norm, register_arrangement
 
 
@@ -30,7 +30,7 @@ class PreNormBlock:
         for slot in self.slots:
             sub = self.spec.names[slot]
             for name, p in getattr(self, slot).named_parameters().items():
-                out[f"{self.spec.prefix}.{sub}.{name}"] = p
+                out[join_name(self.spec.prefix, sub, name)] = p
         return out
 
     def cache_need(self):
@@ -63,6 +63,51 @@ class PreNormBlock:
             stream.push(y, self.residual_scale)
             x = self.norm2.forward(stream)
         stream.push(self.ffn.forward(x, batch), self.residual_scale)
+
+
+@register_arrangement("sandwich_norm")
+class SandwichNormBlock:
+    """x += s * norm1b(mixer(norm1(x))); x += s * norm2b(ffn(norm2(x))): a norm before every sublayer and another on
+    its output before the sum.  A layer may have no feed-forward (no `ffn`, `norm2`, `norm2b` among its parts).  The
+    norms on the outputs give float32 rows, which the next norm's kernel adds to the float32 residual stream."""
+
+    def __init__(self, spec: LayerSpec, ctx: BuildContext):
+        self.spec = spec
+        self.slots = tuple(s for s in ("norm1", "mixer", "norm1b", "norm2", "ffn", "norm2b") if s in spec.parts)
+        if not {"norm1", "mixer", "norm1b"} <= set(self.slots) or (("ffn" in self.slots) != ("norm2" in self.slots)) \
+                or (("ffn" in self.slots) != ("norm2b" in self.slots)):
+            raise ValueError(f"layer {spec.prefix}: a sandwich layer has norm1, mixer, norm1b and, with a feed-forward, norm2 and norm2b")
+        self.norm1 = build_norm(spec.parts["norm1"], ctx)
+        self.mixer = build_mixer(spec.parts["mixer"], ctx)
+        self.norm1b = build_norm(spec.parts["norm1b"], ctx)
+        self.ffn = self.norm2 = self.norm2b = None
+        if "ffn" in self.slots:
+            self.norm2 = build_norm(spec.parts["norm2"], ctx)
+            self.ffn = build_feed_forward(spec.parts["ffn"], ctx)
+            self.norm2b = build_norm(spec.parts["norm2b"], ctx)
+        self.residual_scale = float(spec.residual_scale)
+
+    def named_parameters(self) -> Dict[str, Param]:
+        out: Dict[str, Param] = {}
+        for slot in self.slots:
+            for name, p in getattr(self, slot).named_parameters().items():
+                out[join_name(self.spec.prefix, self.spec.names[slot], name)] = p
+        return out
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def records_mixed_steps(self) -> bool:
+        return bool(getattr(self.mixer, "records_mixed_steps", False)
+                    and (self.ffn is None or getattr(self.ffn, "records_mixed_steps", False)))
+
+    def forward(self, stream: ResidualStream, batch, cache_view) -> None:
+        y = self.mixer.forward(self.norm1.forward(stream), batch, cache_view)
+        stream.push(self.norm1b.apply(y), self.residual_scale)
+        if self.ffn is not None:
+            y = self.ffn.forward(self.norm2.forward(stream), batch)
+            stream.push(self.norm2b.apply(y), self.residual_scale)
 
 
 def build_block(spec: LayerSpec, ctx: BuildContext):

@@ -39,12 +39,13 @@ class OutputHead(Part):
 
 @register_embedding("scaled_lookup")
 class ScaledLookup(Embedding):
-    def __init__(self, vocab_size: int, hidden_size: int, scale: float, ctx: BuildContext):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float, ctx: BuildContext, param_name: str = "weight"):
         self.scale = float(scale)
+        self.param_name = param_name    # "": the table lies under the embedding's own name in a checkpoint
         self.table = torch.empty((int(vocab_size), int(hidden_size)), dtype=ctx.dtype, device=ctx.device)
 
     def named_parameters(self) -> Dict[str, Param]:
-        return {"weight": Param(self.table)}
+        return {self.param_name: Param(self.table)}
 
     def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
         return kernels.embed(token_ids, self.table, self.scale)

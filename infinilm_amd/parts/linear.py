@@ -12,29 +12,57 @@ from typing import Dict, Optional, Sequence
 import torch
 
 from .. import kernels
-from .base import BuildContext, DeferredNorm, NormTail, Param
+from .base import BuildContext, DeferredNorm, NormTail, Param, join_name
 
 
 class FusedLinear:
-    """`out_sizes[i]` rows of the weight belong to the checkpoint tensor `names[i]`."""
+    """`out_sizes[i]` rows of the weight belong to the checkpoint tensor `names[i]`.
+
+    `suffix`: a tensor's name is `names[i]` + "." + suffix ("": the bare name).
+    `out_heads[i]` = (heads, size, padded size): the rows of piece i are heads of `size` rows in a checkpoint, held here
+    as heads of `padded size` rows whose last rows are zeros and stay zeros (`out_sizes[i]` = heads * padded size), so
+    that heads of a size the kernels do not take run as the next size they do.  `in_heads` = (heads, size, padded
+    size): the same for the columns."""
 
     def __init__(self, in_features: int, out_sizes: Sequence[int], names: Sequence[str], bias: bool,
-                 ctx: BuildContext):
+                 ctx: BuildContext, suffix: str = "weight", out_heads: Optional[Sequence] = None,
+                 in_heads: Optional[tuple] = None):
         self.in_features = int(in_features)
         self.out_sizes = [int(s) for s in out_sizes]
         self.names = list(names)
+        self.suffix = suffix
+        self.out_heads = list(out_heads) if out_heads is not None else [None] * len(self.names)
+        self.in_heads = tuple(in_heads) if in_heads is not None and in_heads[1] != in_heads[2] else None
+        for size, oh in zip(self.out_sizes, self.out_heads):
+            if oh is not None and (oh[0] * oh[2] != size or oh[1] > oh[2]):
+                raise ValueError(f"{oh[0]} heads of {oh[1]} filled up to {oh[2]} are not {size} rows")
+        if self.in_heads is not None and (self.in_heads[0] * self.in_heads[2] != self.in_features or bias):
+            raise ValueError("filled-up columns must make up the whole input (and take no bias)")
         n = sum(self.out_sizes)
-        self.weight = torch.empty((n, self.in_features), dtype=ctx.dtype, device=ctx.device)
-        self.bias = torch.empty((n,), dtype=ctx.dtype, device=ctx.device) if bias else None
+        padded = self.in_heads is not None or any(oh is not None and oh[1] != oh[2] for oh in self.out_heads)
+        make = torch.zeros if padded else torch.empty
+        self.weight = make((n, self.in_features), dtype=ctx.dtype, device=ctx.device)
+        self.bias = make((n,), dtype=ctx.dtype, device=ctx.device) if bias else None
         self._frag = {}   # layout -> (version of the weight it was packed from, the weight in fragment order)
 
     def named_parameters(self) -> Dict[str, Param]:
         out: Dict[str, Param] = {}
         row = 0
-        for name, size in zip(self.names, self.out_sizes):
-            out[f"{name}.weight"] = Param(self.weight[row:row + size])
-            if self.bias is not None:
-                out[f"{name}.bias"] = Param(self.bias[row:row + size])
+        for name, size, oh in zip(self.names, self.out_sizes, self.out_heads):
+            w = self.weight[row:row + size]
+            b = self.bias[row:row + size] if self.bias is not None else None
+            if oh is not None and oh[1] != oh[2]:
+                heads, real, pad = oh
+                out[join_name(name, self.suffix)] = Param(w.view(heads, pad, self.in_features)[:, :real], shape=(heads * real, self.in_features))
+                if b is not None:
+                    out[join_name(name, "bias")] = Param(b.view(heads, pad)[:, :real], shape=(heads * real,))
+            elif self.in_heads is not None:
+                heads, real, pad = self.in_heads
+                out[join_name(name, self.suffix)] = Param(w.view(size, heads, pad)[:, :, :real], shape=(size, heads * real))
+            else:
+                out[join_name(name, self.suffix)] = Param(w)
+                if b is not None:
+                    out[join_name(name, "bias")] = Param(b)
             row += size
         return out
 
@@ -66,5 +94,6 @@ class FusedLinear:
 
 
 class Linear(FusedLinear):
-    def __init__(self, in_features: int, out_features: int, name: str, bias: bool, ctx: BuildContext):
-        super().__init__(in_features, [out_features], [name], bias, ctx)
+    def __init__(self, in_features: int, out_features: int, name: str, bias: bool, ctx: BuildContext,
+                 suffix: str = "weight", in_heads: Optional[tuple] = None):
+        super().__init__(in_features, [out_features], [name], bias, ctx, suffix=suffix, in_heads=in_heads)

@@ -46,3 +46,27 @@ class SwiGLU(FeedForward):
             if fused is not None:
                 return fused
         return self.down.forward(kernels.swiglu(gu), allow_parts=True)
+
+
+@register_feed_forward("activation_mlp")
+class ActivationMLP(FeedForward):
+    """down(act(up x)) with one of the kernels' activations (`relu2`: the square of relu, `gelu_tanh`, `silu`, ...).
+    `whole_output`: the result comes as one [T, hidden] tensor in the activations' dtype, for an arrangement that norms
+    it before it is added."""
+    records_mixed_steps = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str, bias: bool, ctx: BuildContext,
+                 names=("up_proj", "down_proj"), suffix: str = "weight", whole_output: bool = False):
+        kernels._act(activation)
+        self.activation = activation
+        self.whole_output = bool(whole_output)
+        self.up = Linear(hidden_size, intermediate_size, names[0], bias, ctx, suffix=suffix)
+        self.down = Linear(intermediate_size, hidden_size, names[1], bias, ctx, suffix=suffix)
+
+    def named_parameters(self) -> Dict[str, Param]:
+        out = dict(self.up.named_parameters())
+        out.update(self.down.named_parameters())
+        return out
+
+    def forward(self, x, batch) -> torch.Tensor:
+        return self.down.forward(kernels.activation(self.up.forward(x), self.activation), allow_parts=not self.whole_output)

@@ -20,17 +20,23 @@ from .registry import register_norm
 class RMSNorm(Norm):
     takes_frag_request = True
 
-    def __init__(self, size: int, eps: float, ctx: BuildContext):
+    def __init__(self, size: int, eps: float, ctx: BuildContext, param_name: str = "weight"):
         self.size = int(size)
         self.eps = float(eps)
         self.dtype = ctx.dtype
+        self.param_name = param_name    # "": the weight lies under the norm's own name in a checkpoint
         self.weight = torch.empty((self.size,), dtype=ctx.dtype, device=ctx.device)
 
     def _set_weight(self, t: torch.Tensor) -> None:
         self.weight = t
 
     def named_parameters(self) -> Dict[str, Param]:
-        return {"weight": Param(self.weight, keep_f32=True, replace=self._set_weight, neutral=1.0)}
+        return {self.param_name: Param(self.weight, keep_f32=True, replace=self._set_weight, neutral=1.0)}
+
+    def apply(self, x: torch.Tensor, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+        """The norm of rows that are not the residual stream (a branch's output normed before it is added): sums in
+        float32, the result in `out_dtype`."""
+        return kernels.group_norm_gate(x, self.weight, self.eps, 1, out_dtype=out_dtype)
 
     def tail(self, stream: ResidualStream, scale: float, rows: int):
         if stream.pending is not None or self.dtype != torch.bfloat16 or rows > kernels.TAIL_MAX_ROWS:

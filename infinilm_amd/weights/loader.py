@@ -21,6 +21,8 @@ from typing import Iterator, List, Tuple
 
 import torch
 
+from ..parts.base import join_name
+
 
 class WeightError(RuntimeError):
     """Missing, unexpected or wrongly shaped tensors; lists all of them."""
@@ -68,7 +70,8 @@ def load_weights(model, model_dir: str) -> None:
 
 def load_state_dict(model, tensors) -> None:
     params = model.named_parameters()
-    head_name = f"{model.spec.head.name}.weight"
+    head_name = join_name(model.spec.head.name, "weight")
+    embed_names = [join_name(model.spec.embed_name, n) for n in model.embedding.named_parameters()]
     seen, unexpected, wrong, other = set(), [], [], []
     items = tensors.items() if isinstance(tensors, dict) else tensors
     for name, t in items:
@@ -80,8 +83,8 @@ def load_state_dict(model, tensors) -> None:
             unexpected.append(name)
             continue
         seen.add(name)
-        if tuple(t.shape) != tuple(p.tensor.shape):
-            wrong.append(f"{name}: checkpoint {tuple(t.shape)}, model {tuple(p.tensor.shape)}")
+        if tuple(t.shape) != tuple(p.shape):
+            wrong.append(f"{name}: checkpoint {tuple(t.shape)}, model {tuple(p.shape)}")
             continue
         if not (t.dtype.is_floating_point or t.dtype in (torch.int8, torch.int16, torch.int32, torch.int64, torch.uint8)):
             other.append(f"{name}: unsupported dtype {t.dtype}")
@@ -93,10 +96,10 @@ def load_state_dict(model, tensors) -> None:
         if p.keep_f32 and t.dtype == torch.float32 and p.tensor.dtype != torch.float32:
             p.replace(t.to(p.tensor.device))
         else:
-            p.tensor.copy_(t.to(p.tensor.dtype))
+            p.store(t)
     missing = [n for n in params if n not in seen]
     if head_name in missing and model.spec.head.tie_to_embedding_when_missing \
-            and f"{model.spec.embed_name}.weight" in seen:
+            and all(n in seen for n in embed_names):
         model.tie_head_to_embedding()
         missing.remove(head_name)
     if missing or unexpected or wrong or other:

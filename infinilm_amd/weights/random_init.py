@@ -37,7 +37,7 @@ def random_state_dict(config: dict, seed: int, std: float = 0.02, norm_init: str
         if tied and name == f"{meta.spec.head.name}.weight":
             continue
         g = torch.Generator().manual_seed((int(seed) * 1000003 + i) & 0x7fffffffffff)
-        t = torch.randn(tuple(p.tensor.shape), generator=g, dtype=torch.float32) * std
+        t = torch.randn(tuple(p.shape), generator=g, dtype=torch.float32) * std
         if norm_init == "one_plus" and p.neutral != 0.0:
             t = t + p.neutral
         out[name] = t.to(store).contiguous()
