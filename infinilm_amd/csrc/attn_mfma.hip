@@ -46,13 +46,21 @@ __device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
 
+// A raw score under a cap: the raw score whose scaled value is cap * tanh(scaled score / cap), so that what follows
+// (the scale inside the exponent's multiply-add) stays as it is.  capq = cap / scale; capq <= 0: no cap.
+// tanh(x) = 1 - 2 / (e^(2x) + 1): exact at both ends (e^(2x) = 0 or infinity).
+__device__ __forceinline__ float att_cap(float raw, float capq, float icapq) {
+    const float e = __builtin_amdgcn_exp2f(raw * icapq * 2.885390081777927f);
+    return capq * (1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f));
+}
+
 template <int D16>
 __global__ void __launch_bounds__(ATT_WAVES * 64, 2)
 attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __restrict__ ws_ml,
                  const bf16* __restrict__ q, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                  const int* __restrict__ block_tables, const int* __restrict__ seg,
                  const int* __restrict__ pos, const int* __restrict__ rows, int nh, int nkv, int page,
-                 int max_blocks, int q_stride, int out_stride, float scale_log2e, int window, int nsplit, int span) {
+                 int max_blocks, int q_stride, int out_stride, float scale_log2e, float capq, int window, int nsplit, int span) {
     constexpr int D = D16 * 16;
     constexpr int KS = (D + 31) / 32;
     __shared__ float sm_acc[ATT_WAVES][D16][64][4];
@@ -145,7 +153,8 @@ attn_mfma_kernel(bf16* __restrict__ out, float* __restrict__ ws_acc, float* __re
                 _Pragma("unroll") for (int e = 0; e < 4; ++e) {                                            \
                     const int key = kb_ + qg * 8 + tau * 4 + e;                                            \
                     const bool ok = key >= kbeg_ && key < kend_;                                           \
-                    const float v = ok ? s[tau][e] * scale_log2e : NEG_BIG;                                \
+                    const float raw = capq > 0.f ? att_cap(s[tau][e], capq, 1.0f / capq) : s[tau][e];      \
+                    const float v = ok ? raw * scale_log2e : NEG_BIG;                                      \
                     sv[tau * 4 + e] = v;                                                                   \
                     mx = fmaxf(mx, v);                                                                     \
                 }                                                                                          \
@@ -395,7 +404,7 @@ __global__ void __launch_bounds__(256, 2)
 attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ kc,
                  const bf16* __restrict__ vc, const int* __restrict__ block_tables, const int* __restrict__ seg,
                  const int* __restrict__ pos, const int* __restrict__ tiles, int nh, int nkv, int page,
-                 int max_blocks, int q_stride, int out_stride, float scale_log2e, int window, int pair_base) {
+                 int max_blocks, int q_stride, int out_stride, float scale_log2e, float capq, int window, int pair_base) {
     constexpr int D = D16 * 16;
     constexpr int KS = (D + 31) / 32;
     // K rows [key][d] and V rows [d][key] in LDS, read in 16-byte pieces by 16 rows x 4 lane groups.
@@ -648,6 +657,12 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
             /* scores become exponents relative to the reference point, in place */                       \
             float lm[ATT_NT];                                                                              \
             bool over = false;                                                                             \
+            if (capq > 0.f) {                                                                              \
+                const float icapq = 1.0f / capq;                                                           \
+                _Pragma("unroll") for (int j = 0; j < ATT_NT; ++j)                                         \
+                    _Pragma("unroll") for (int tau = 0; tau < 2; ++tau)                                    \
+                        _Pragma("unroll") for (int e = 0; e < 4; ++e) S_[j][tau][e] = att_cap(S_[j][tau][e], capq, icapq); \
+            }                                                                                              \
             _Pragma("unroll") for (int j = 0; j < ATT_NT; ++j) {                                           \
                 const bool unset = mc[j] < 0.5f * NEG_BIG;   /* no key seen yet: exponents relative to 0 */ \
                 const float nm = unset ? 0.f : -mc[j];                                                     \
@@ -820,7 +835,7 @@ attn_tile_kernel(bf16* __restrict__ out, const bf16* __restrict__ q, const bf16*
 #pragma unroll
                 for (int tau = 0; tau < 2; ++tau)
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) sv[j][tau * 4 + e] = s[sub][j][tau][e];
+                    for (int e = 0; e < 4; ++e) sv[j][tau * 4 + e] = capq > 0.f ? att_cap(s[sub][j][tau][e], capq, 1.0f / capq) : s[sub][j][tau][e];
                 if (!full) {
 #pragma unroll
                     for (int i = 0; i < 8; ++i) {
@@ -923,7 +938,7 @@ extern "C" int ilm_attn_tile_tokens() { return ATT_TT; }
 extern "C" int ilm_attn_tile(void* out, const void* q, const void* kc, const void* vc, const void* block_tables,
                              const void* seg, const void* pos, const void* tiles, int n_tiles, int nh, int nkv,
                              int d, int page, int max_blocks, int q_stride, int out_stride, float scale,
-                             int window, hipStream_t stream) {
+                             int window, float softcap, hipStream_t stream) {
     ILM_REQUIRE(n_tiles > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_tile: bad sizes");
     ILM_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "attn_tile: head size %d is not a multiple of 16 up to 128", d);
     ILM_REQUIRE(page % 16 == 0 && page > 0, "attn_tile: page size %d is not a multiple of 16", page);
@@ -933,11 +948,12 @@ extern "C" int ilm_attn_tile(void* out, const void* q, const void* kc, const voi
     ILM_REQUIRE(nkv * HG <= 65535, "attn_tile: grid too large");
     dim3 grid(n_tiles, nkv * HG);
     const float sl2 = scale * 1.4426950408889634f;
+    const float capq = softcap > 0.f ? softcap / scale : 0.f;
     const int cus = ilm_num_cus();
     const long long n_items = (long long)n_tiles * nkv * HG;
     const int pair_base = (n_items > cus && n_items <= 2 * cus) ? cus : 0;
 #define AT_ARGS (bf16*)out, (const bf16*)q, (const bf16*)kc, (const bf16*)vc, (const int*)block_tables, (const int*)seg, \
-                (const int*)pos, (const int*)tiles, nh, nkv, page, max_blocks, q_stride, out_stride, sl2, window, pair_base
+                (const int*)pos, (const int*)tiles, nh, nkv, page, max_blocks, q_stride, out_stride, sl2, capq, window, pair_base
 #define AT_CASE(D16)                                                                   \
     case D16:                                                                          \
         if (page % ATT_TK == 0) attn_tile_kernel<D16, true><<<grid, 256, 0, stream>>>(AT_ARGS);  \
@@ -960,7 +976,7 @@ static int attn_mfma_launch(void* out, void* ws_acc, void* ws_ml, const void* q,
                             const void* vc, const void* block_tables, const void* seg, const void* pos,
                             const void* rows, int T_, int nh, int nkv, int d, int page, int max_blocks,
                             int q_stride, int out_stride, float scale, int window, int nsplit, int span,
-                            hipStream_t stream) {
+                            float softcap, hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attn_mfma: bad head counts nh=%d nkv=%d", nh, nkv);
     ILM_REQUIRE(d % 16 == 0 && d >= 16 && d <= 128, "attn_mfma: head size %d is not a multiple of 16 up to 128", d);
     ILM_REQUIRE(page % 16 == 0 && page > 0, "attn_mfma: page size %d is not a multiple of 16", page);
@@ -972,12 +988,13 @@ static int attn_mfma_launch(void* out, void* ws_acc, void* ws_ml, const void* q,
     ILM_REQUIRE(nkv * HG <= 65535 && nsplit <= ATT_MERGE_MAX_CHUNKS, "attn_mfma: at most %d chunks, got %d", ATT_MERGE_MAX_CHUNKS, nsplit);
     dim3 grid(T_, nkv * HG, nsplit);
     const float sl2 = scale * 1.4426950408889634f;
+    const float capq = softcap > 0.f ? softcap / scale : 0.f;
 #define AM_CASE(D16)                                                                                           \
     case D16:                                                                                                  \
         attn_mfma_kernel<D16><<<grid, ATT_WAVES * 64, 0, stream>>>(                                            \
             (bf16*)out, (float*)ws_acc, (float*)ws_ml, (const bf16*)q, (const bf16*)kc, (const bf16*)vc,      \
             (const int*)block_tables, (const int*)seg, (const int*)pos, (const int*)rows, nh, nkv, page,      \
-            max_blocks, q_stride, out_stride, sl2, window, nsplit, span);                                      \
+            max_blocks, q_stride, out_stride, sl2, capq, window, nsplit, span);                                      \
         break
     switch (d / 16) {
         AM_CASE(1); AM_CASE(2); AM_CASE(3); AM_CASE(4); AM_CASE(5); AM_CASE(6); AM_CASE(7); AM_CASE(8);
@@ -1003,9 +1020,9 @@ extern "C" int ilm_attn_mfma(void* out, void* ws_acc, void* ws_ml, const void* q
                              const void* vc, const void* block_tables, const void* seg, const void* pos,
                              const void* rows, int T_, int nh, int nkv, int d, int page, int max_blocks,
                              int q_stride, int out_stride, float scale, int window, int nsplit, int span,
-                             hipStream_t stream) {
+                             float softcap, hipStream_t stream) {
     return attn_mfma_launch(out, ws_acc, ws_ml, q, kc, vc, block_tables, seg, pos, rows, T_, nh, nkv, d, page, max_blocks,
-                            q_stride, out_stride, scale, window, nsplit, span, stream);
+                            q_stride, out_stride, scale, window, nsplit, span, softcap, stream);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1065,5 +1082,5 @@ extern "C" int ilm_attn_mfma_static(void* out, const void* q, const void* kc, co
         ws_ml = base + acc_floats;   // d is a multiple of 16: 64-byte aligned
     }
     return attn_mfma_launch(out, ws_acc, ws_ml, q, kc, vc, block_tables, seg, pos, rows, T_, nh, nkv, d, page, max_blocks,
-                            q_stride, out_stride, scale, window, nsplit, span, stream);
+                            q_stride, out_stride, scale, window, nsplit, span, 0.f, stream);
 }

@@ -696,7 +696,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         raise KernelError("per-token metadata does not match the number of tokens")
     out = torch.empty((T, nh * d), dtype=q.dtype, device=q.device)
     if (q.dtype == BF16 and not FORCE_BASIC and d % 16 == 0 and d <= 128 and page % 16 == 0 and q.stride(0) % 8 == 0
-            and max_total_len is not None and not softcap > 0.0):
+            and max_total_len is not None):
         n_single = T
         rows = None
         if tiles is not None and tiles.numel() > 0:
@@ -705,7 +705,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
             _run("ilm_attn_tile", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                  block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), tiles.data_ptr(),
                  tiles.numel() // 2, nh, nkv, d, page, block_tables.shape[1], q.stride(0), out.stride(0), float(scale),
-                 int(window), _stream())
+                 int(window), float(softcap), _stream())
             if single_rows is None or single_rows.numel() == 0:
                 return out
             _i32(single_rows, "single_rows")
@@ -720,7 +720,7 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         _run("ilm_attn_mfma", out.data_ptr(), _ptr(ws_acc), _ptr(ws_ml), q.data_ptr(), k_cache.data_ptr(),
              v_cache.data_ptr(), block_tables.data_ptr(), seg_of_token.data_ptr(), positions.data_ptr(), _ptr(rows),
              n_single, nh, nkv, d, page, block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window),
-             nsplit, span, _stream())
+             nsplit, span, float(softcap), _stream())
         return out
     bound = block_tables.shape[1] * page if max_total_len is None else min(int(max_total_len), block_tables.shape[1] * page)
     if (q.dtype == F32 and not FORCE_BASIC and d % 16 == 0 and d <= 256 and page % 4 == 0 and q.stride(0) % 4 == 0

@@ -76,7 +76,7 @@ def _run(L, c, span, static):
     else:
         ws_acc = torch.empty((n * nh * nsplit * d,), dtype=torch.float32, device=DEV)
         ws_ml = torch.empty((n * nh * nsplit * 2,), dtype=torch.float32, device=DEV)
-        rc = L.ilm_attn_mfma(ptr(out), ptr(ws_acc), ptr(ws_ml), *common, *tail)
+        rc = L.ilm_attn_mfma(ptr(out), ptr(ws_acc), ptr(ws_ml), *common, *tail[:-1], 0.0, stream)   # (no cap on the scores)
     torch.cuda.synchronize()
     return rc, out
 
