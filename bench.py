@@ -50,6 +50,10 @@ def main() -> int:
     ap.add_argument("--prefill-only", action="store_true", help="only the prefill measurement (for profiling)")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 32 / 64 points, the prefill and the 32-bit record")
     ap.add_argument("--no-fp32", action="store_true", help="skip the 32-bit record (bfloat16 runs only)")
+    ap.add_argument("--designs", action="store_true",
+                    help="instead of the default workload: prefill and decode throughput of the Kekevik design beside MiniCPM4 "
+                         "at equal layer sizes (random weights), with the time and the roofline share of every kernel")
+    ap.add_argument("--design-shapes", default="1024,4096", help="widths to compare with --designs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (N>1 is not run)")
@@ -61,6 +65,9 @@ def main() -> int:
 
     require_gpu("cuda:0")
     lib.load()
+    if args.designs:
+        print(json.dumps(compare_designs(args)))
+        return 0
     FULL_LAYERS = 32
     cfg = config_8b(args.layers)
     record = measure(args, cfg, args.dtype, FULL_LAYERS, full=True)
@@ -71,6 +78,126 @@ def main() -> int:
                           "prefill_ms": f["prefill"]["ms"], "prefill_frac": f["prefill"]["frac"]}
     print(json.dumps(record))
     return 0
+
+
+def compare_designs(args) -> dict:
+    """Kekevik beside MiniCPM4 at equal width, layers, heads, head size and feed-forward parameters: prefill of
+    `--prefill-tokens` tokens in one step, decode at batch 8 and 64 over `--context` tokens (recorded steps), and for
+    every kernel entry point its calls, its time a call in eager steps and, where one bound names it, the share of that
+    bound it reaches: bytes it must move over the HBM peak, or floating-point work over the vector float32 peak."""
+    import torch
+    from infinilm_amd import kernels
+    from infinilm_amd.engine.loading import build_model, make_runner
+    from infinilm_amd.engine.step import StepEntry
+    from infinilm_amd.sampling import Sampler, SamplingParams
+    from infinilm_amd.weights import fill_random_
+    sys.path.insert(0, os.path.join(ROOT, "examples"))
+    from shapes import kekevik_shape
+
+    layers = 8 if args.layers == 32 else args.layers
+    T, ctx, ps = args.prefill_tokens, min(args.context, 2048), args.page_size
+    out = {"metric": "prefill and decode tokens/s, Kekevik beside MiniCPM4 at equal layer sizes", "dtype": "bf16", "layers": layers,
+           "prefill_tokens": T, "context": ctx, "data": "synthetic: random weights and token ids, random-filled cache", "shapes": {}}
+    sampler, greedy = Sampler(0), SamplingParams(top_k=1)
+    gen = torch.Generator().manual_seed(7)
+    for width in [int(w) for w in args.design_shapes.split(",")]:
+        heads, d, kv, V = width // 128, 128, 2, 32768
+        cfgs = {
+            "minicpm4": {"architectures": ["MiniCPMForCausalLM"], "model_type": "minicpm", "torch_dtype": "bfloat16", "rope_theta": 10000.0,
+                         "num_hidden_layers": layers, "hidden_size": width, "num_attention_heads": heads, "num_key_value_heads": kv,
+                         "head_dim": d, "intermediate_size": 4 * width, "vocab_size": V, "max_position_embeddings": 32768,
+                         "rms_norm_eps": 1e-6, "tie_word_embeddings": True},
+            "kekevik": kekevik_shape(width, heads, d, kv, layers, V, 6 * width)}
+        rec = {}
+        for name, cfg in cfgs.items():
+            model = build_model(cfg, "bfloat16", "cuda:0")
+            fill_random_(model, seed=0, std=0.02, norm_init="one_plus")
+            Hs = model.spec.hidden_size
+            params = sum(p.tensor.numel() for p in model.named_parameters().values())
+            r = {"parameters": params}
+            for graph in (True, False):
+                runner = make_runner(model, num_pages=64 * (-(-(ctx + 1) // ps)) + -(-T // ps) + 4, page_size=ps, max_requests=65,
+                                     enable_graph=graph)
+                cache = runner.cache
+                for e in cache.k:
+                    cache.k[e].normal_(0, 1.0)
+                    cache.v[e].normal_(0, 1.0)
+
+                def prefill(passes):
+                    prompt = torch.randint(0, V, (T,), generator=gen).tolist()
+                    times = []
+                    for i in range(passes):
+                        cache.admit("p")
+                        torch.cuda.synchronize()
+                        t0 = time.perf_counter()
+                        sampler.sample(runner.step([StepEntry("p", prompt, [T - 1])]), [(greedy, 0, 0)])
+                        torch.cuda.synchronize()
+                        times.append(time.perf_counter() - t0)
+                        cache.release("p")
+                    return sorted(times[1:])[len(times[1:]) // 2]
+
+                def decode(batch, steps, warmup):
+                    ids = [f"d{i}" for i in range(batch)]
+                    for rid in ids:
+                        cache.admit(rid)
+                        cache.reserve(rid, ctx - steps - warmup)
+                        cache.commit(rid, ctx - steps - warmup)
+                    toks = torch.randint(0, V, (batch,), generator=gen).tolist()
+                    for i in range(steps + warmup):
+                        if i == warmup:
+                            torch.cuda.synchronize()
+                            t0 = time.perf_counter()
+                        toks = sampler.sample(runner.step([StepEntry(rid, [t], [0]) for rid, t in zip(ids, toks)]),
+                                              [(greedy, j, 0) for j in range(batch)])
+                    torch.cuda.synchronize()
+                    dt = (time.perf_counter() - t0) / steps
+                    for rid in ids:
+                        cache.release(rid)
+                    return dt
+
+                if graph:
+                    pt = prefill(5)
+                    r["prefill_tok_s"] = round(T / pt, 1)
+                    r["prefill_ms"] = round(pt * 1e3, 3)
+                    for b in (8, 64):
+                        dt = decode(b, max(8, args.steps // 2), args.warmup)
+                        r[f"decode_b{b}_tok_s"] = round(b / dt, 1)
+                        r[f"decode_b{b}_ms"] = round(dt * 1e3, 4)
+                else:   # eager steps with a pair of events around every launch: the kernels' own times
+                    kernels.enable_timing(True)
+                    prefill(2)
+                    kernels.timing_report()
+                    prefill(2)
+                    rep_p = kernels.timing_report()
+                    decode(64, 4, 2)
+                    kernels.timing_report()
+                    decode(64, 4, 0)
+                    rep_d = kernels.timing_report()
+                    kernels.enable_timing(False)
+                    r["kernels_prefill_us"] = {k: [v["calls"], v["mean_us"]] for k, v in sorted(rep_p.items())}
+                    r["kernels_decode_b64_us"] = {k: [v["calls"], v["mean_us"]] for k, v in sorted(rep_d.items())}
+                    # bounds of the kernels that the design adds, and of the attention kernels beside them
+                    us = lambda rep, k: rep[k]["mean_us"] * 1e-6 if k in rep else None
+                    share = {}
+                    state = heads * d * d * 4          # a head's state x heads (key size = value size = state entries = d here)
+                    kvb = 2 * kv * d * 2               # cached bytes a token
+                    if us(rep_d, "ilm_decay_scan"):
+                        share["decay_scan decode (state read + written / HBM peak)"] = round(64 * 2 * state / us(rep_d, "ilm_decay_scan") / HBM_PEAK, 4)
+                        share["decay_scan prefill (4 dk dv flops a token and head / float32 vector peak)"] = round(
+                            4.0 * T * heads * d * d / us(rep_p, "ilm_decay_scan") / FLOP_PEAK["fp32"], 4)
+                    if us(rep_d, "ilm_attn_mfma"):
+                        share["attention decode (cache read / HBM peak)"] = round(64 * ctx * kvb / us(rep_d, "ilm_attn_mfma") / HBM_PEAK, 4)
+                    if us(rep_p, "ilm_attn_tile"):
+                        share["attention prefill (4 d flops a visible key and head / bf16 matrix peak)"] = round(
+                            4.0 * T * T / 2 * heads * d / us(rep_p, "ilm_attn_tile") / FLOP_PEAK["bf16"], 4)
+                    r["roofline_share"] = share
+                del runner, cache
+                torch.cuda.empty_cache()
+            rec[name] = r
+            del model
+            torch.cuda.empty_cache()
+        out["shapes"][str(width)] = rec
+    return out
 
 
 def measure(args, cfg, dtype, FULL_LAYERS, full):

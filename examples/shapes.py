@@ -39,3 +39,18 @@ def shape_config(name: str, layers: int = 0) -> dict:
     if layers > 0:
         cfg["num_hidden_layers"] = int(layers)
     return cfg
+
+
+def kekevik_shape(width: int, heads: int, head_dim: int, kv_heads: int, layers: int, vocab: int, ff: int) -> dict:
+    """A Kekevik configuration with the layer sizes of a transformer of this width: the four layer kinds in turn
+    (retention, lightning, two side-by-side layers), `heads` heads of `head_dim` everywhere, a state space of
+    heads * head_dim channels with 128 state entries a head, `ff` inner units of the feed-forward."""
+    decay = [1.0 - 2.0 ** -(5 + (7 * h) // max(heads, 1)) for h in range(heads)]
+    lin = {"heads": heads, "dim": head_dim, "vdim": head_dim, "decay": decay}
+    par = {"left": {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+                    "softcap": 50.0, "q_temp": {"coef": 0.1, "every": 1024}},
+           "right": {"heads": heads, "vdim": head_dim, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1},
+           "left_scale": 1.0, "right_scale": 1.0}
+    kinds = [("retention", dict(lin, rot={"dims": head_dim, "base": 10000.0})), ("lightning", lin), ("parallel", par), ("parallel", par)]
+    return {"architecture": "Kekevik", "vocab": vocab, "width": width, "embedding": {"scale": 12.0}, "norm": {"eps": 1e-6},
+            "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]}

@@ -46,10 +46,33 @@ unary_kernel(void* __restrict__ out, const void* __restrict__ in, int n, int out
     stf(out, out_dt, (size_t)t * out_stride + j, act_f(ldf(in, in_dt, (size_t)t * in_stride + j), kind));
 }
 
+// bfloat16 rows, eight elements a thread (16-byte accesses): n and the strides multiples of 8, rows 16 bytes aligned
+__global__ void __launch_bounds__(256)
+unary_vec_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ in, int n, int out_stride, int in_stride, int kind) {
+    const int t = blockIdx.y;
+    const int j = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (j >= n) return;
+    uint16_t a[8], r[8];
+    *reinterpret_cast<uint4*>(a) = *reinterpret_cast<const uint4*>(in + (size_t)t * in_stride + j);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) r[e] = __builtin_bit_cast(uint16_t, (__bf16)act_f(bf16_bits_to_f32(a[e]), kind));
+    *reinterpret_cast<uint4*>(out + (size_t)t * out_stride + j) = *reinterpret_cast<uint4*>(r);
+}
+
 extern "C" int ilm_unary(void* out, const void* in, int T_, int n, int out_stride, int in_stride, int kind, int out_dt,
                          int in_dt, hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && n > 0 && T_ <= 65535 * 32768, "unary: bad sizes T=%d n=%d", T_, n);
     ILM_REQUIRE(kind >= 0 && kind <= RC_ACT_GELU_TANH, "unary: unknown activation %d", kind);
+    if (out_dt == ILM_DTYPE_BF16 && in_dt == ILM_DTYPE_BF16 && n % 8 == 0 && out_stride % 8 == 0 && in_stride % 8 == 0
+        && ((uintptr_t)out & 15) == 0 && ((uintptr_t)in & 15) == 0) {
+        for (int t0 = 0; t0 < T_; t0 += 65535) {
+            const int rows = T_ - t0 < 65535 ? T_ - t0 : 65535;
+            unary_vec_kernel<<<dim3((n / 8 + 255) / 256, rows), 256, 0, stream>>>(
+                (uint16_t*)out + (size_t)t0 * out_stride, (const uint16_t*)in + (size_t)t0 * in_stride, n, out_stride, in_stride, kind);
+        }
+        ILM_LAUNCH_CHECK("unary");
+        return 0;
+    }
     for (int t0 = 0; t0 < T_; t0 += 65535) {
         const int rows = T_ - t0 < 65535 ? T_ - t0 : 65535;
         const size_t eo = out_dt == ILM_DTYPE_F32 ? 4 : 2, ei = in_dt == ILM_DTYPE_F32 ? 4 : 2;
@@ -121,126 +144,376 @@ extern "C" int ilm_lin_prep(void* out, const void* in, const void* pos, const vo
 // a_t comes per head (decay_h) or per token and head (decay_t [T, heads]); b_t (kscale_t [T, heads]) and skip
 // (skip_h [heads]) may be absent.  Head h reads the q and k of group h / q_div.
 // Requests are the segments of the step: seg_offsets [R + 1] rows, state_in / state_out [R] pool rows.
+//
+// Long segments (portions of prompts) are cut into pieces of `piece` tokens that run side by side, in three launches:
+//   SC_LOCAL    every piece runs its tokens from a zero state and leaves that local state, and the product of its
+//               decays, in a workspace slot;
+//   (combine)   per segment, piece after piece: the state at a piece's start = decay product of the piece before x the
+//               state at that piece's start + its local state, written over the local states; the state after the last
+//               piece goes to the pool;
+//   SC_FROM     every piece runs its tokens again from its start state and writes the outputs.
+// Twice the arithmetic of one pass, and as many blocks as the step has pieces.  Piece p of segment r has the slot
+// floor(first row of r / piece) + r + p: slots of different segments never meet, and floor(T / piece) + R slots hold all.
+// A block finds its (segment, piece) from its slot by bisection over the segments' first slots.
 // ------------------------------------------------------------------------------------------
 #define SC_NK 8
+#define SC_WHOLE 0
+#define SC_LOCAL 1
+#define SC_FROM 2
 
+// the segment whose slots hold slot s (-1: none), its piece p
+__device__ __forceinline__ int sc_find(const int* __restrict__ seg_offsets, int R, int piece, int s, int& p) {
+    int lo = 0, hi = R - 1;     // the last segment whose first slot is <= s
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (seg_offsets[mid] / piece + mid <= s) lo = mid; else hi = mid - 1;
+    }
+    p = s - (seg_offsets[lo] / piece + lo);
+    const int len = seg_offsets[lo + 1] - seg_offsets[lo];
+    return (p >= 0 && p * piece < len) ? lo : -1;
+}
+
+template <int MODE, int VC>   // VC: value columns a thread (the q and k a thread loads serve all of them)
 __global__ void __launch_bounds__(256)
 decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__ q, const float* __restrict__ k,
                   int qk_stride, int q_div, const float* __restrict__ v, int v_stride,
                   const float* __restrict__ decay_h, const float* __restrict__ decay_t,
                   const float* __restrict__ kscale_t, const float* __restrict__ skip_h, float* __restrict__ pool,
                   const int* __restrict__ state_in, const int* __restrict__ state_out,
-                  const int* __restrict__ seg_offsets, int heads, int dk, int dv, int KP) {
-    const int r = blockIdx.z, h = blockIdx.y;
-    const int t0 = seg_offsets[r], t1 = seg_offsets[r + 1];
-    if (t0 >= t1) return;
-    const int VT = 256 / KP;
-    const int kp = threadIdx.x % KP, vc = blockIdx.x * VT + threadIdx.x / KP;
-    const bool vok = vc < dv;
-    const size_t hs = (size_t)dk * dv;                       // floats of a head's state
-    const size_t row_in = ((size_t)state_in[r] * heads + h) * hs, row_out = ((size_t)state_out[r] * heads + h) * hs;
-    float S[SC_NK];
-#pragma unroll
-    for (int i = 0; i < SC_NK; ++i) {
-        const int ki = i * KP + kp;
-        S[i] = (vok && ki < dk) ? pool[row_in + (size_t)vc * dk + ki] : 0.f;
+                  const int* __restrict__ seg_offsets, int heads, int dk, int dv, int KP, int R, int piece,
+                  float* __restrict__ ws_state, float* __restrict__ ws_decay) {
+    const int h = blockIdx.y;
+    int r, t0, t1, slot = 0;
+    if (MODE == SC_WHOLE) {
+        r = blockIdx.z;
+        t0 = seg_offsets[r];
+        t1 = seg_offsets[r + 1];
+        if (t0 >= t1) return;
+    } else {
+        int p;
+        slot = blockIdx.z;
+        r = sc_find(seg_offsets, R, piece, slot, p);
+        if (r < 0) return;
+        t0 = seg_offsets[r] + p * piece;
+        t1 = min(t0 + piece, seg_offsets[r + 1]);
     }
+    const int VT = 256 / KP;                                 // column groups a block
+    const int kp = threadIdx.x % KP, vc0 = (blockIdx.x * VT + threadIdx.x / KP) * VC;
+    const size_t hs = (size_t)dk * dv;                       // floats of a head's state
+    const float* src = MODE == SC_WHOLE ? pool + ((size_t)state_in[r] * heads + h) * hs
+                                        : ws_state + ((size_t)slot * heads + h) * hs;
+    float S[VC][SC_NK];
+#pragma unroll
+    for (int c = 0; c < VC; ++c)
+#pragma unroll
+        for (int i = 0; i < SC_NK; ++i) {
+            const int ki = i * KP + kp;
+            S[c][i] = (MODE != SC_LOCAL && vc0 + c < dv && ki < dk) ? src[(size_t)(vc0 + c) * dk + ki] : 0.f;
+        }
     const int qoff = (h / q_div) * dk;
     const float a_h = decay_h != nullptr ? decay_h[h] : 1.0f;
     const float skip = skip_h != nullptr ? skip_h[h] : 0.f;
-    float qn[SC_NK], kn[SC_NK], vn, an, bn;
+    float qn[SC_NK], kn[SC_NK], vn[VC], an, bn;
+    float aprod = 1.0f;
 #define SC_LOAD(T_)                                                                              \
     {                                                                                            \
         const float* qr = q + (size_t)(T_) * qk_stride + qoff;                                   \
         const float* kr = k + (size_t)(T_) * qk_stride + qoff;                                   \
         _Pragma("unroll") for (int i = 0; i < SC_NK; ++i) {                                      \
             const int ki = i * KP + kp;                                                          \
-            qn[i] = ki < dk ? qr[ki] : 0.f;                                                      \
+            if (MODE != SC_LOCAL) qn[i] = ki < dk ? qr[ki] : 0.f;                                \
             kn[i] = ki < dk ? kr[ki] : 0.f;                                                      \
         }                                                                                        \
-        vn = vok ? v[(size_t)(T_) * v_stride + (size_t)h * dv + vc] : 0.f;                       \
+        _Pragma("unroll") for (int c = 0; c < VC; ++c)                                           \
+            vn[c] = vc0 + c < dv ? v[(size_t)(T_) * v_stride + (size_t)h * dv + vc0 + c] : 0.f;  \
         an = decay_t != nullptr ? decay_t[(size_t)(T_) * heads + h] : a_h;                       \
         bn = kscale_t != nullptr ? kscale_t[(size_t)(T_) * heads + h] : 1.0f;                    \
     }
     SC_LOAD(t0)
     for (int t = t0; t < t1; ++t) {
-        float qc[SC_NK], kc[SC_NK];
+        float qc[SC_NK], kc[SC_NK], vcur[VC];
+        const float a = an, b = bn;
 #pragma unroll
         for (int i = 0; i < SC_NK; ++i) {
-            qc[i] = qn[i];
-            kc[i] = kn[i];
+            if (MODE != SC_LOCAL) qc[i] = qn[i];
+            kc[i] = kn[i] * b;
         }
-        const float vcur = vn, a = an, bv = bn * vn;
+#pragma unroll
+        for (int c = 0; c < VC; ++c) vcur[c] = vn[c];
         if (t + 1 < t1) SC_LOAD(t + 1)
-        float acc = 0.f;
+        float acc[VC];
 #pragma unroll
-        for (int i = 0; i < SC_NK; ++i) {
-            S[i] = fmaf(a, S[i], kc[i] * bv);
-            acc = fmaf(S[i], qc[i], acc);
+        for (int c = 0; c < VC; ++c) {
+            acc[c] = 0.f;
+#pragma unroll
+            for (int i = 0; i < SC_NK; ++i) {
+                S[c][i] = fmaf(a, S[c][i], kc[i] * vcur[c]);
+                if (MODE != SC_LOCAL) acc[c] = fmaf(S[c][i], qc[i], acc[c]);
+            }
         }
-        for (int off = 1; off < KP; off <<= 1) acc += __shfl_xor(acc, off, 64);
-        if (kp == 0 && vok) o[(size_t)t * o_stride + (size_t)h * dv + vc] = fmaf(skip, vcur, acc);
+        if (MODE == SC_LOCAL) {
+            aprod *= a;
+        } else {
+#pragma unroll
+            for (int c = 0; c < VC; ++c) {
+                for (int off = 1; off < KP; off <<= 1) acc[c] += __shfl_xor(acc[c], off, 64);
+                if (kp == 0 && vc0 + c < dv) o[(size_t)t * o_stride + (size_t)h * dv + vc0 + c] = fmaf(skip, vcur[c], acc[c]);
+            }
+        }
     }
 #undef SC_LOAD
-    if (vok) {
+    if (MODE == SC_FROM) return;
+    float* dst = MODE == SC_WHOLE ? pool + ((size_t)state_out[r] * heads + h) * hs : ws_state + ((size_t)slot * heads + h) * hs;
+#pragma unroll
+    for (int c = 0; c < VC; ++c)
 #pragma unroll
         for (int i = 0; i < SC_NK; ++i) {
             const int ki = i * KP + kp;
-            if (ki < dk) pool[row_out + (size_t)vc * dk + ki] = S[i];
+            if (vc0 + c < dv && ki < dk) dst[(size_t)(vc0 + c) * dk + ki] = S[c][i];
         }
+    if (MODE == SC_LOCAL && blockIdx.x == 0 && threadIdx.x == 0) ws_decay[(size_t)slot * heads + h] = aprod;
+}
+
+// The pieces' form of the kernel above (SC_LOCAL, SC_FROM): a token's q, k, v, decay and scale reach the threads through
+// LDS in tiles of TB tokens that the block loads together, the next tile on its way from memory while this one is
+// computed (one barrier a tile), instead of every thread loading its own entries token by token: a wave then waits for
+// memory once a tile, not once a token.  Thread (kp, column group) owns the SC_NK consecutive state entries
+// kp * SC_NK ... of its VC columns.  LDS: 2 buffers x TB x (2 dkp + columns + 2) floats, dkp = KP * SC_NK.
+template <int MODE, int VC>
+__global__ void __launch_bounds__(256)
+decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __restrict__ q, const float* __restrict__ k,
+                        int qk_stride, int q_div, const float* __restrict__ v, int v_stride,
+                        const float* __restrict__ decay_h, const float* __restrict__ decay_t,
+                        const float* __restrict__ kscale_t, const float* __restrict__ skip_h,
+                        const int* __restrict__ seg_offsets, int heads, int dk, int dv, int KP, int R, int piece, int TB,
+                        float* __restrict__ ws_state, float* __restrict__ ws_decay) {
+    extern __shared__ float lds[];
+    const int h = blockIdx.y, slot = blockIdx.z;
+    int p;
+    const int r = sc_find(seg_offsets, R, piece, slot, p);
+    if (r < 0) return;
+    const int t0 = seg_offsets[r] + p * piece, t1 = min(t0 + piece, seg_offsets[r + 1]);
+    const int VT = 256 / KP, cols = VT * VC, dkp = KP * SC_NK;
+    const int kp = threadIdx.x % KP, cl = (threadIdx.x / KP) * VC;   // first column of the thread inside the block
+    const int vb = blockIdx.x * cols;                                 // first column of the block
+    const size_t hs = (size_t)dk * dv;
+    float* st = ws_state + ((size_t)slot * heads + h) * hs;
+    const int per = TB * (2 * dkp + cols + 2);                        // floats of one buffer: q | k | v | a | b
+    float S[VC][SC_NK];
+#pragma unroll
+    for (int c = 0; c < VC; ++c)
+#pragma unroll
+        for (int i = 0; i < SC_NK; ++i) {
+            const int ki = kp * SC_NK + i, vc = vb + cl + c;
+            S[c][i] = (MODE == SC_FROM && vc < dv && ki < dk) ? st[(size_t)vc * dk + ki] : 0.f;
+        }
+    const int qoff = (h / q_div) * dk;
+    const float a_h = decay_h != nullptr ? decay_h[h] : 1.0f;
+    const float skip = skip_h != nullptr ? skip_h[h] : 0.f;
+    float rq[8], rk[8], rv[8], ra = 1.f, rb = 1.f;     // a tile on its way: TB * dkp <= 2048 and TB * cols <= 2048
+#define SCT_FETCH(T0_)                                                                                       \
+    {                                                                                                        \
+        _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                                      \
+            const int idx = threadIdx.x + i * 256, tt = idx / dkp, ki = idx % dkp;                           \
+            const bool ok = idx < TB * dkp && (T0_) + tt < t1 && ki < dk;                                    \
+            const size_t at = (size_t)((T0_) + tt) * qk_stride + qoff + ki;                                  \
+            rq[i] = (MODE == SC_FROM && ok) ? q[at] : 0.f;                                                   \
+            rk[i] = ok ? k[at] : 0.f;                                                                        \
+        }                                                                                                    \
+        _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                                      \
+            const int idx = threadIdx.x + i * 256, tt = idx / cols, c = idx % cols;                          \
+            const bool ok = idx < TB * cols && (T0_) + tt < t1 && vb + c < dv;                               \
+            rv[i] = ok ? v[(size_t)((T0_) + tt) * v_stride + (size_t)h * dv + vb + c] : 0.f;                 \
+        }                                                                                                    \
+        if (threadIdx.x < TB && (T0_) + threadIdx.x < t1) {                                                  \
+            ra = decay_t != nullptr ? decay_t[(size_t)((T0_) + threadIdx.x) * heads + h] : a_h;              \
+            rb = kscale_t != nullptr ? kscale_t[(size_t)((T0_) + threadIdx.x) * heads + h] : 1.0f;           \
+        }                                                                                                    \
     }
+#define SCT_STORE(BUF_)                                                                                      \
+    {                                                                                                        \
+        float* b_ = lds + (BUF_) * per;                                                                      \
+        _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                                      \
+            const int idx = threadIdx.x + i * 256;                                                           \
+            if (idx < TB * dkp) {                                                                            \
+                b_[idx] = rq[i];                                                                             \
+                b_[TB * dkp + idx] = rk[i];                                                                  \
+            }                                                                                                \
+            if (idx < TB * cols) b_[2 * TB * dkp + idx] = rv[i];                                             \
+        }                                                                                                    \
+        if (threadIdx.x < TB) {                                                                              \
+            b_[TB * (2 * dkp + cols) + threadIdx.x] = ra;                                                    \
+            b_[TB * (2 * dkp + cols + 1) + threadIdx.x] = rb;                                                \
+        }                                                                                                    \
+    }
+    SCT_FETCH(t0)
+    SCT_STORE(0)
+    __syncthreads();
+    float aprod = 1.0f;
+    int buf = 0;
+    for (int tb = t0; tb < t1; tb += TB, buf ^= 1) {
+        const bool more = tb + TB < t1;
+        if (more) SCT_FETCH(tb + TB)
+        const float* b_ = lds + buf * per;
+        const int n = min(TB, t1 - tb);
+        for (int tt = 0; tt < n; ++tt) {
+            float qc[SC_NK], kc[SC_NK], vcur[VC];
+            const float a = b_[TB * (2 * dkp + cols) + tt], bsc = b_[TB * (2 * dkp + cols + 1) + tt];
+#pragma unroll
+            for (int i4 = 0; i4 < SC_NK; i4 += 4) {
+                if (MODE == SC_FROM) {
+                    const float4 t4 = *reinterpret_cast<const float4*>(b_ + tt * dkp + kp * SC_NK + i4);
+                    qc[i4] = t4.x; qc[i4 + 1] = t4.y; qc[i4 + 2] = t4.z; qc[i4 + 3] = t4.w;
+                }
+                const float4 u4 = *reinterpret_cast<const float4*>(b_ + TB * dkp + tt * dkp + kp * SC_NK + i4);
+                kc[i4] = u4.x * bsc; kc[i4 + 1] = u4.y * bsc; kc[i4 + 2] = u4.z * bsc; kc[i4 + 3] = u4.w * bsc;
+            }
+#pragma unroll
+            for (int c = 0; c < VC; ++c) vcur[c] = b_[2 * TB * dkp + tt * cols + cl + c];
+            float acc[VC];
+#pragma unroll
+            for (int c = 0; c < VC; ++c) {
+                acc[c] = 0.f;
+#pragma unroll
+                for (int i = 0; i < SC_NK; ++i) {
+                    S[c][i] = fmaf(a, S[c][i], kc[i] * vcur[c]);
+                    if (MODE == SC_FROM) acc[c] = fmaf(S[c][i], qc[i], acc[c]);
+                }
+            }
+            if (MODE == SC_LOCAL) {
+                aprod *= a;
+            } else {
+#pragma unroll
+                for (int c = 0; c < VC; ++c) {
+                    for (int off = 1; off < KP; off <<= 1) acc[c] += __shfl_xor(acc[c], off, 64);
+                    if (kp == 0 && vb + cl + c < dv)
+                        o[(size_t)(tb + tt) * o_stride + (size_t)h * dv + vb + cl + c] = fmaf(skip, vcur[c], acc[c]);
+                }
+            }
+        }
+        if (more) SCT_STORE(buf ^ 1)
+        __syncthreads();
+    }
+#undef SCT_FETCH
+#undef SCT_STORE
+    if (MODE == SC_FROM) return;
+#pragma unroll
+    for (int c = 0; c < VC; ++c)
+#pragma unroll
+        for (int i = 0; i < SC_NK; ++i) {
+            const int ki = kp * SC_NK + i, vc = vb + cl + c;
+            if (vc < dv && ki < dk) st[(size_t)vc * dk + ki] = S[c][i];
+        }
+    if (blockIdx.x == 0 && threadIdx.x == 0) ws_decay[(size_t)slot * heads + h] = aprod;
+}
+
+// per (segment, head), piece after piece: ws_state[slot] <- the state at the piece's start; the pool gets the last state
+__global__ void __launch_bounds__(256)
+decay_scan_combine_kernel(float* __restrict__ ws_state, const float* __restrict__ ws_decay, float* __restrict__ pool,
+                          const int* __restrict__ state_in, const int* __restrict__ state_out,
+                          const int* __restrict__ seg_offsets, int heads, int hs, int piece) {
+    const int r = blockIdx.z, h = blockIdx.y, e = blockIdx.x * 256 + threadIdx.x;
+    const int t0 = seg_offsets[r], len = seg_offsets[r + 1] - t0;
+    if (len <= 0 || e >= hs) return;
+    const int pieces = (len + piece - 1) / piece, base = t0 / piece + r;
+    float S = pool[((size_t)state_in[r] * heads + h) * hs + e];
+    for (int p = 0; p < pieces; ++p) {
+        float* at = ws_state + ((size_t)(base + p) * heads + h) * hs + e;
+        const float local = *at;
+        *at = S;
+        S = fmaf(ws_decay[(size_t)(base + p) * heads + h], S, local);
+    }
+    pool[((size_t)state_out[r] * heads + h) * hs + e] = S;
 }
 
 extern "C" int ilm_decay_scan_max_dk() { return SC_NK * 64; }
 
+// piece == 0: one pass, a block a (segment, head, columns).  piece > 0: segments in pieces of that many tokens (see
+// above); ws_state holds (T / piece + R) * heads * dk * dv floats, ws_decay (T / piece + R) * heads.
 extern "C" int ilm_decay_scan(void* o, int o_stride, const void* q, const void* k, int qk_stride, int q_div, const void* v,
                               int v_stride, const void* decay_h, const void* decay_t, const void* kscale_t,
                               const void* skip_h, void* pool, const void* state_in, const void* state_out,
-                              const void* seg_offsets, int R, int heads, int dk, int dv, hipStream_t stream) {
-    ILM_REQUIRE(R > 0 && heads > 0 && dk > 0 && dv > 0, "decay_scan: bad sizes");
+                              const void* seg_offsets, int R, int heads, int dk, int dv, int T_, int piece, void* ws_state,
+                              void* ws_decay, hipStream_t stream) {
+    ILM_REQUIRE(R > 0 && heads > 0 && dk > 0 && dv > 0 && T_ > 0, "decay_scan: bad sizes");
     ILM_REQUIRE(dk <= SC_NK * 64, "decay_scan: %d state entries a column, at most %d", dk, SC_NK * 64);
     ILM_REQUIRE(q_div > 0 && heads % q_div == 0, "decay_scan: %d heads do not divide into groups of %d", heads, q_div);
     ILM_REQUIRE((decay_h != nullptr) != (decay_t != nullptr), "decay_scan: a decay per head or per token, one of them");
     ILM_REQUIRE(R <= 65535 && heads <= 65535, "decay_scan: too many requests or heads");
+    ILM_REQUIRE(piece >= 0 && (piece == 0 || (ws_state != nullptr && ws_decay != nullptr)), "decay_scan: pieces need a workspace");
     int KP = 1;
     while (KP * SC_NK < dk) KP <<= 1;
     const int VT = 256 / KP;
-    dim3 grid((dv + VT - 1) / VT, heads, R);
-    decay_scan_kernel<<<grid, 256, 0, stream>>>((float*)o, o_stride, (const float*)q, (const float*)k, qk_stride, q_div,
-                                                (const float*)v, v_stride, (const float*)decay_h, (const float*)decay_t,
-                                                (const float*)kscale_t, (const float*)skip_h, (float*)pool,
-                                                (const int*)state_in, (const int*)state_out, (const int*)seg_offsets, heads,
-                                                dk, dv, KP);
-    ILM_LAUNCH_CHECK("decay_scan");
+#define SC_ARGS (float*)o, o_stride, (const float*)q, (const float*)k, qk_stride, q_div, (const float*)v, v_stride,              \
+                (const float*)decay_h, (const float*)decay_t, (const float*)kscale_t, (const float*)skip_h, (float*)pool,        \
+                (const int*)state_in, (const int*)state_out, (const int*)seg_offsets, heads, dk, dv, KP, R, piece,              \
+                (float*)ws_state, (float*)ws_decay
+    // four columns a thread where that still leaves two blocks a compute unit (long prompts in pieces, large batches):
+    // a thread's loads of q and k then serve four columns; one column a thread where blocks are few (small batches)
+    const int cus = ilm_num_cus();
+    if (piece == 0) {
+        const int g4 = (dv + 4 * VT - 1) / (4 * VT);
+        if ((long)g4 * heads * R >= 2L * cus && dv >= 4) decay_scan_kernel<SC_WHOLE, 4><<<dim3(g4, heads, R), 256, 0, stream>>>(SC_ARGS);
+        else decay_scan_kernel<SC_WHOLE, 1><<<dim3((dv + VT - 1) / VT, heads, R), 256, 0, stream>>>(SC_ARGS);
+        ILM_LAUNCH_CHECK("decay_scan");
+        return 0;
+    }
+    const int slots = T_ / piece + R;
+    ILM_REQUIRE(slots <= 65535, "decay_scan: %d pieces in a step, at most 65535", slots);
+    const int g4 = (dv + 4 * VT - 1) / (4 * VT);
+    const bool four = (long)g4 * heads * (T_ / piece + 1) >= 2L * cus && dv >= 4;
+    const int cols = VT * (four ? 4 : 1), dkp = KP * SC_NK;
+    int TB = 16;
+    while (TB > 1 && (TB * dkp > 2048 || TB * cols > 2048)) TB >>= 1;
+    const size_t shm = (size_t)2 * TB * (2 * dkp + cols + 2) * sizeof(float);
+    dim3 grid(four ? g4 : (dv + VT - 1) / VT, heads, slots);
+#define SCT_ARGS (float*)o, o_stride, (const float*)q, (const float*)k, qk_stride, q_div, (const float*)v, v_stride,             \
+                 (const float*)decay_h, (const float*)decay_t, (const float*)kscale_t, (const float*)skip_h,                    \
+                 (const int*)seg_offsets, heads, dk, dv, KP, R, piece, TB, (float*)ws_state, (float*)ws_decay
+    if (four) decay_scan_tiled_kernel<SC_LOCAL, 4><<<grid, 256, shm, stream>>>(SCT_ARGS);
+    else decay_scan_tiled_kernel<SC_LOCAL, 1><<<grid, 256, shm, stream>>>(SCT_ARGS);
+    ILM_LAUNCH_CHECK("decay_scan (local states)");
+    decay_scan_combine_kernel<<<dim3((dk * dv + 255) / 256, heads, R), 256, 0, stream>>>(
+        (float*)ws_state, (const float*)ws_decay, (float*)pool, (const int*)state_in, (const int*)state_out,
+        (const int*)seg_offsets, heads, dk * dv, piece);
+    ILM_LAUNCH_CHECK("decay_scan (combine)");
+    if (four) decay_scan_tiled_kernel<SC_FROM, 4><<<grid, 256, shm, stream>>>(SCT_ARGS);
+    else decay_scan_tiled_kernel<SC_FROM, 1><<<grid, 256, shm, stream>>>(SCT_ARGS);
+    ILM_LAUNCH_CHECK("decay_scan (outputs)");
+#undef SCT_ARGS
+#undef SC_ARGS
     return 0;
 }
 
 // ------------------------------------------------------------------------------------------
-// RMS norm in groups with an optional gate, one wave a (row, group):
+// RMS norm in groups with an optional gate, one wave (groups up to 512 elements) or one block a (row, group):
 //   y = x * act(gate)            (gate_before)
 //   y = y / sqrt(mean_group(y^2) + eps) * w       (w may be absent)
 //   y = y * act(gate)            (otherwise)
 // Sums run over a group in an order that depends on its size only.
 // ------------------------------------------------------------------------------------------
+template <int LANES>   // threads an item: 64 (four items a block) or 256
 __global__ void __launch_bounds__(256)
 group_norm_gate_kernel(void* __restrict__ out, const void* __restrict__ x, const void* __restrict__ gate,
                        const void* __restrict__ w, int rows, int n, int groups, int x_stride, int gate_stride,
                        int out_stride, float eps, int gate_act, int gate_before, int out_dt, int x_dt, int gate_dt, int w_dt) {
-    const int item = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-    if (item >= rows * groups) return;
+    __shared__ float red[4];
+    const int item = LANES == 64 ? blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
+    const int lane = LANES == 64 ? (threadIdx.x & 63) : threadIdx.x;
+    if (item >= rows * groups) return;     // (whole waves; with 256 lanes an item every block has one)
     const int t = item / groups, g = item % groups, gs = n / groups;
     const size_t xb = (size_t)t * x_stride + (size_t)g * gs, gb = (size_t)t * gate_stride + (size_t)g * gs;
     const size_t ob = (size_t)t * out_stride + (size_t)g * gs;
     const bool pre = gate != nullptr && gate_before;
     float ss = 0.f;
-    for (int j = lane; j < gs; j += 64) {
+    for (int j = lane; j < gs; j += LANES) {
         float y = ldf(x, x_dt, xb + j);
         if (pre) y *= act_f(ldf(gate, gate_dt, gb + j), gate_act);
         ss = fmaf(y, y, ss);
     }
-    ss = wave_sum(ss);
+    ss = LANES == 64 ? wave_sum(ss) : block_sum<4>(ss, red);
     const float rstd = 1.0f / sqrtf(ss / (float)gs + eps);
-    for (int j = lane; j < gs; j += 64) {
+    for (int j = lane; j < gs; j += LANES) {
         float y = ldf(x, x_dt, xb + j);
         if (pre) y *= act_f(ldf(gate, gate_dt, gb + j), gate_act);
         y *= rstd;
@@ -255,9 +528,14 @@ extern "C" int ilm_group_norm_gate(void* out, const void* x, const void* gate, c
                                    int out_dt, int x_dt, int gate_dt, int w_dt, hipStream_t stream) {
     ILM_REQUIRE(rows > 0 && n > 0 && groups > 0 && n % groups == 0, "group_norm_gate: %d elements do not divide into %d groups", n, groups);
     ILM_REQUIRE((long)rows * groups < (1L << 31) - 4, "group_norm_gate: too many rows");
-    const int blocks = (int)(((long)rows * groups + 3) / 4);
-    group_norm_gate_kernel<<<blocks, 256, 0, stream>>>(out, x, gate, w, rows, n, groups, x_stride, gate_stride, out_stride, eps,
-                                                      gate_act, gate_before, out_dt, x_dt, gate_dt, w_dt);
+    if (n / groups > 512) {
+        group_norm_gate_kernel<256><<<rows * groups, 256, 0, stream>>>(out, x, gate, w, rows, n, groups, x_stride, gate_stride,
+                                                                       out_stride, eps, gate_act, gate_before, out_dt, x_dt, gate_dt, w_dt);
+    } else {
+        const int blocks = (int)(((long)rows * groups + 3) / 4);
+        group_norm_gate_kernel<64><<<blocks, 256, 0, stream>>>(out, x, gate, w, rows, n, groups, x_stride, gate_stride, out_stride,
+                                                               eps, gate_act, gate_before, out_dt, x_dt, gate_dt, w_dt);
+    }
     ILM_LAUNCH_CHECK("group_norm_gate");
     return 0;
 }
@@ -266,39 +544,51 @@ extern "C" int ilm_group_norm_gate(void* out, const void* x, const void* gate, c
 // Short causal convolution over the tokens of each request, per channel, with bias and activation:
 //   y[t, c] = act(b[c] + sum_i w[c, i] * x[t - (taps - 1) + i, c]),   the last tap is the token's own input.
 // Inputs before a request's first token of this step come from its state row (the last taps - 1 inputs of the
-// steps before, oldest first; zeros for a new request); the row is then written anew.  One thread a (request,
-// channel) walks the request's tokens with the window in registers, so a state entry has one reader and writer.
+// steps before, oldest first; zeros for a new request).  One thread a (token, channel); a second launch, one thread a
+// (request, channel), then writes the state row anew from the old row and the step's inputs (it reads what it
+// overwrites into registers first, and no other thread touches its entries).
 // ------------------------------------------------------------------------------------------
 #define CV_MAX_TAPS 8
 
 __global__ void __launch_bounds__(256)
 causal_conv_kernel(float* __restrict__ y, const void* __restrict__ x, const void* __restrict__ w, const void* __restrict__ b,
-                   float* __restrict__ pool, const int* __restrict__ state_in, const int* __restrict__ state_out,
+                   const float* __restrict__ pool, const int* __restrict__ state_in, const int* __restrict__ seg_of_token,
                    const int* __restrict__ seg_offsets, int C, int taps, int x_stride, int y_stride, int act, int x_dt, int w_dt) {
-    const int r = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    const int t = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
-    const int t0 = seg_offsets[r], t1 = seg_offsets[r + 1];
-    if (t0 >= t1) return;
-    float win[CV_MAX_TAPS], wt[CV_MAX_TAPS];
-    const size_t sin = (size_t)state_in[r] * (taps - 1) * C, sout = (size_t)state_out[r] * (taps - 1) * C;
+    const int r = seg_of_token[t];
+    const int j = t - seg_offsets[r];                       // the token's place in its segment
+    const size_t sin = (size_t)state_in[r] * (taps - 1) * C;
+    float s = b != nullptr ? ldf(b, w_dt, c) : 0.f;
 #pragma unroll
     for (int i = 0; i < CV_MAX_TAPS; ++i) {
-        wt[i] = i < taps ? ldf(w, w_dt, (size_t)c * taps + i) : 0.f;
-        win[i] = i < taps - 1 ? pool[sin + (size_t)i * C + c] : 0.f;
-    }
-    const float bias = b != nullptr ? ldf(b, w_dt, c) : 0.f;
-    const float w_last = ldf(w, w_dt, (size_t)c * taps + taps - 1);   // the token's own tap
-    for (int t = t0; t < t1; ++t) {
-        const float xv = ldf(x, x_dt, (size_t)t * x_stride + c);
-        float s = bias;
-#pragma unroll
-        for (int i = 0; i < CV_MAX_TAPS; ++i) {
-            if (i < taps - 1) s = fmaf(wt[i], win[i], s);
+        if (i < taps) {
+            const int back = taps - 1 - i;                  // tap i reads the input `back` tokens before
+            const float xv = back <= j ? ldf(x, x_dt, (size_t)(t - back) * x_stride + c)
+                                       : pool[sin + (size_t)(taps - 1 - (back - j)) * C + c];
+            s = fmaf(ldf(w, w_dt, (size_t)c * taps + i), xv, s);
         }
-        s = fmaf(w_last, xv, s);
-        y[(size_t)t * y_stride + c] = act_f(s, act);
+    }
+    y[(size_t)t * y_stride + c] = act_f(s, act);
+}
+
+__global__ void __launch_bounds__(256)
+causal_conv_state_kernel(const void* __restrict__ x, float* __restrict__ pool, const int* __restrict__ state_in,
+                         const int* __restrict__ state_out, const int* __restrict__ seg_offsets, int C, int taps,
+                         int x_stride, int x_dt) {
+    const int r = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int t0 = seg_offsets[r], len = seg_offsets[r + 1] - t0;
+    if (len <= 0) return;
+    const size_t sin = (size_t)state_in[r] * (taps - 1) * C, sout = (size_t)state_out[r] * (taps - 1) * C;
+    float win[CV_MAX_TAPS];
 #pragma unroll
-        for (int i = 0; i < CV_MAX_TAPS - 1; ++i) win[i] = (i + 1 < taps - 1) ? win[i + 1] : (i == taps - 2 ? xv : win[i]);
+    for (int i = 0; i < CV_MAX_TAPS; ++i) {
+        // entry i of the new row: the input taps - 1 - i tokens before the segment's end
+        const int back = taps - 1 - i;
+        win[i] = 0.f;
+        if (i < taps - 1) win[i] = back <= len ? ldf(x, x_dt, (size_t)(t0 + len - back) * x_stride + c)
+                                               : pool[sin + (size_t)(i + len) * C + c];
     }
 #pragma unroll
     for (int i = 0; i < CV_MAX_TAPS; ++i)
@@ -308,14 +598,24 @@ causal_conv_kernel(float* __restrict__ y, const void* __restrict__ x, const void
 extern "C" int ilm_causal_conv_max_taps() { return CV_MAX_TAPS; }
 
 extern "C" int ilm_causal_conv(void* y, const void* x, const void* w, const void* b, void* pool, const void* state_in,
-                               const void* state_out, const void* seg_offsets, int R, int C, int taps, int x_stride,
-                               int y_stride, int act, int x_dt, int w_dt, hipStream_t stream) {
-    ILM_REQUIRE(R > 0 && C > 0 && R <= 65535, "causal_conv: bad sizes");
+                               const void* state_out, const void* seg_of_token, const void* seg_offsets, int T_, int R, int C,
+                               int taps, int x_stride, int y_stride, int act, int x_dt, int w_dt, hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && R > 0 && C > 0 && R <= 65535, "causal_conv: bad sizes");
     ILM_REQUIRE(taps >= 1 && taps <= CV_MAX_TAPS, "causal_conv: %d taps, at most %d", taps, CV_MAX_TAPS);
-    causal_conv_kernel<<<dim3((C + 255) / 256, R), 256, 0, stream>>>((float*)y, x, w, b, (float*)pool, (const int*)state_in,
-                                                                     (const int*)state_out, (const int*)seg_offsets, C, taps,
-                                                                     x_stride, y_stride, act, x_dt, w_dt);
+    for (int t0 = 0; t0 < T_; t0 += 65535) {
+        const int rows = T_ - t0 < 65535 ? T_ - t0 : 65535;
+        causal_conv_kernel<<<dim3((C + 255) / 256, rows), 256, 0, stream>>>(
+            (float*)y + (size_t)t0 * y_stride, (const char*)x + (size_t)t0 * x_stride * (x_dt == ILM_DTYPE_F32 ? 4 : 2), w, b,
+            (const float*)pool, (const int*)state_in, (const int*)seg_of_token + t0, (const int*)seg_offsets, C, taps, x_stride,
+            y_stride, act, x_dt, w_dt);
+    }
     ILM_LAUNCH_CHECK("causal_conv");
+    if (taps > 1) {
+        causal_conv_state_kernel<<<dim3((C + 255) / 256, R), 256, 0, stream>>>(x, (float*)pool, (const int*)state_in,
+                                                                                (const int*)state_out, (const int*)seg_offsets, C,
+                                                                                taps, x_stride, x_dt);
+        ILM_LAUNCH_CHECK("causal_conv_state");
+    }
     return 0;
 }
 
@@ -416,9 +716,30 @@ weighted_sum_kernel(void* __restrict__ out, const void* __restrict__ x, const vo
     stf(out, out_dt, i, fmaf(a, ldf(x, x_dt, i), b * ldf(y, y_dt, i)));
 }
 
+__global__ void __launch_bounds__(256)
+weighted_sum_vec_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ y, long n,
+                        float a, float b) {
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i >= n) return;
+    uint16_t p[8], q[8], r[8];
+    *reinterpret_cast<uint4*>(p) = *reinterpret_cast<const uint4*>(x + i);
+    *reinterpret_cast<uint4*>(q) = *reinterpret_cast<const uint4*>(y + i);
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+        r[e] = __builtin_bit_cast(uint16_t, (__bf16)fmaf(a, bf16_bits_to_f32(p[e]), b * bf16_bits_to_f32(q[e])));
+    *reinterpret_cast<uint4*>(out + i) = *reinterpret_cast<uint4*>(r);
+}
+
 extern "C" int ilm_weighted_sum(void* out, const void* x, const void* y, long n, float a, float b, int out_dt, int x_dt,
                                 int y_dt, hipStream_t stream) {
     ILM_REQUIRE(n > 0 && (n + 255) / 256 < (1L << 31), "weighted_sum: bad size");
+    if (out_dt == ILM_DTYPE_BF16 && x_dt == ILM_DTYPE_BF16 && y_dt == ILM_DTYPE_BF16 && n % 8 == 0 && ((uintptr_t)out & 15) == 0
+        && ((uintptr_t)x & 15) == 0 && ((uintptr_t)y & 15) == 0) {
+        weighted_sum_vec_kernel<<<(unsigned)((n / 8 + 255) / 256), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)x,
+                                                                                     (const uint16_t*)y, n, a, b);
+        ILM_LAUNCH_CHECK("weighted_sum");
+        return 0;
+    }
     weighted_sum_kernel<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(out, x, y, n, a, b, out_dt, x_dt, y_dt);
     ILM_LAUNCH_CHECK("weighted_sum");
     return 0;

@@ -1016,6 +1016,8 @@ def gemm_frag_tail(x: FragRows, fw: FragWeight, bias: Optional[torch.Tensor], al
 # ---- mixers with a fixed-size state, and the small steps around them -------------------------------------------------
 ACTIVATIONS = {"none": 0, "silu": 1, "sigmoid": 2, "relu2": 3, "gelu_tanh": 4}
 SCAN_MAX_KEY_DIM = 512      # most state entries a value column of the recurrence (ilm_decay_scan_max_dk())
+SCAN_PIECE = int(os.environ.get("INFINILM_AMD_SCAN_PIECE", "64"))        # tokens a piece of a long segment (0: never cut)
+SCAN_PIECE_FROM = int(os.environ.get("INFINILM_AMD_SCAN_PIECE_FROM", "129"))   # segments from this length on are cut
 CONV_MAX_TAPS = 8           # most taps of the short convolution (ilm_causal_conv_max_taps())
 
 
@@ -1067,12 +1069,15 @@ def linear_attention_inputs(qkv: torch.Tensor, positions: Optional[torch.Tensor]
 def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, dk: int, dv: int, groups: int,
                pool: torch.Tensor, state_in: torch.Tensor, state_out: torch.Tensor, seg_offsets: torch.Tensor, segments: int,
                decay_h: Optional[torch.Tensor] = None, decay_t: Optional[torch.Tensor] = None,
-               kscale_t: Optional[torch.Tensor] = None, skip_h: Optional[torch.Tensor] = None) -> torch.Tensor:
+               kscale_t: Optional[torch.Tensor] = None, skip_h: Optional[torch.Tensor] = None,
+               max_len: Optional[int] = None) -> torch.Tensor:
     """S_t = a_t S_(t-1) + (b_t k_t) v_t^T, o_t = S_t^T q_t + skip_h v_t for every head of every segment, token by token,
     all in float32.  q, k: [T, groups*dk] (views with one row stride; head h reads group h // (heads/groups)), v [T, heads*dv];
     a per head (`decay_h` [heads]) or per token (`decay_t` [T, heads]); b `kscale_t` [T, heads] or absent.  `pool`
     [rows, heads, dv, dk] holds the states: segment r starts from row state_in[r] and leaves its state in row state_out[r].
-    Returns o [T, heads*dv]."""
+    `max_len`: a bound on the segments' lengths known on the host; from SCAN_PIECE_FROM tokens on, segments are cut
+    into pieces of SCAN_PIECE tokens that run side by side (two passes and a combination of the pieces' states; the
+    result differs from the single pass by rounding).  Returns o [T, heads*dv]."""
     _dev(q, k, v, pool, state_in, state_out, seg_offsets, decay_h, decay_t, kscale_t, skip_h)
     for t, nm in ((q, "q"), (k, "k"), (v, "v")):
         _rows(t, nm)
@@ -1097,9 +1102,16 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, dk
     if (decay_h is None) == (decay_t is None):
         raise KernelError("the recurrence takes a decay per head or per token, one of them")
     o = torch.empty((T, heads * dv), dtype=F32, device=v.device)
+    piece, ws_state, ws_decay = 0, None, None
+    if SCAN_PIECE > 0 and max_len is not None and max_len >= SCAN_PIECE_FROM and T // SCAN_PIECE + int(segments) <= 65535:
+        piece = SCAN_PIECE
+        slots = T // piece + int(segments)
+        ws_state = torch.empty((slots * heads * dv * dk,), dtype=F32, device=v.device)
+        ws_decay = torch.empty((slots * heads,), dtype=F32, device=v.device)
     _run("ilm_decay_scan", o.data_ptr(), o.stride(0), q.data_ptr(), k.data_ptr(), q.stride(0), heads // groups, v.data_ptr(),
          v.stride(0), _ptr(decay_h), _ptr(decay_t), _ptr(kscale_t), _ptr(skip_h), pool.data_ptr(), state_in.data_ptr(),
-         state_out.data_ptr(), seg_offsets.data_ptr(), int(segments), heads, dk, dv, _stream())
+         state_out.data_ptr(), seg_offsets.data_ptr(), int(segments), heads, dk, dv, T, piece, _ptr(ws_state), _ptr(ws_decay),
+         _stream())
     return o
 
 
@@ -1127,14 +1139,17 @@ def group_norm_gate(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
 
 
 def causal_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], pool: torch.Tensor,
-                state_in: torch.Tensor, state_out: torch.Tensor, seg_offsets: torch.Tensor, segments: int,
-                act: str = "silu") -> torch.Tensor:
+                state_in: torch.Tensor, state_out: torch.Tensor, seg_of_token: torch.Tensor, seg_offsets: torch.Tensor,
+                segments: int, act: str = "silu") -> torch.Tensor:
     """y[t, c] = act(bias[c] + sum_i weight[c, i] x[t - taps + 1 + i, c]) over the tokens of each segment; what lies
     before a segment's first row comes from its row of `pool` [rows, taps - 1, channels] (float32, oldest first), which
     is then written anew (row state_out[r]).  float32 result [T, channels]."""
-    _dev(x, weight, bias, pool, state_in, state_out, seg_offsets)
+    _dev(x, weight, bias, pool, state_in, state_out, seg_of_token, seg_offsets)
     _rows(x, "x")
     T, C = x.shape
+    _i32(seg_of_token, "seg_of_token")
+    if seg_of_token.numel() != T:
+        raise KernelError("seg_of_token must have one entry a token")
     if weight.dim() != 2 or weight.shape[0] != C or not weight.is_contiguous() or not 1 <= weight.shape[1] <= CONV_MAX_TAPS:
         raise KernelError(f"convolution weight {tuple(weight.shape)} must be [{C}, taps <= {CONV_MAX_TAPS}]")
     taps = weight.shape[1]
@@ -1148,8 +1163,8 @@ def causal_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
         raise KernelError("state rows and offsets must cover every segment")
     y = torch.empty((T, C), dtype=F32, device=x.device)
     _run("ilm_causal_conv", y.data_ptr(), x.data_ptr(), weight.data_ptr(), _ptr(bias), pool.data_ptr(), state_in.data_ptr(),
-         state_out.data_ptr(), seg_offsets.data_ptr(), int(segments), C, taps, x.stride(0), y.stride(0), _act(act), _dt(x),
-         _dt(weight), _stream())
+         state_out.data_ptr(), seg_of_token.data_ptr(), seg_offsets.data_ptr(), T, int(segments), C, taps, x.stride(0),
+         y.stride(0), _act(act), _dt(x), _dt(weight), _stream())
     return y
 
 

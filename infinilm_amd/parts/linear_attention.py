@@ -73,7 +73,8 @@ class DecayLinearAttention(Mixer):
         rows = self.proj.forward(x)                                    # [T, q | k | v | g]
         f = kernels.linear_attention_inputs(rows, batch.positions, self.freq, H, dk, dv, self.rd, self.activation, self.k_scale)
         o = kernels.decay_scan(f[:, :H * dk], f[:, H * dk:2 * H * dk], f[:, 2 * H * dk:], H, dk, dv, H, view.pool,
-                               view.state_in, view.state_out, batch.seg_offsets, view.state_in.numel(), decay_h=self.decay)
+                               view.state_in, view.state_out, batch.seg_offsets, view.state_in.numel(), decay_h=self.decay,
+                               max_len=batch.max_q_len)
         y = kernels.group_norm_gate(o, self.norm_w, self.eps, self.norm_groups, gate=rows[:, 2 * H * dk + H * dv:],
                                     gate_act=self.gate_act, out_dtype=self.dtype)
         return self.o_proj.forward(y)

@@ -72,11 +72,11 @@ class SelectiveStateSpace(Mixer):
         segments = ssm_view.state_in.numel()
         u = self.in_proj.forward(x)                              # [T, z | x | B | C | dt]
         c = kernels.causal_conv(u[:, inner:inner + self.C], self.conv_w, self.conv_b, conv_view.pool, conv_view.state_in,
-                                conv_view.state_out, batch.seg_offsets, segments, "silu")          # float32 [T, x | B | C]
+                                conv_view.state_out, batch.seg_of_token, batch.seg_offsets, segments, "silu")          # float32 [T, x | B | C]
         dt, decay = kernels.ssm_steps(u[:, inner + self.C:], self.dt_bias, self.a_log)
         y = kernels.decay_scan(c[:, inner + GN:], c[:, inner:inner + GN], c[:, :inner], self.H, self.N, self.dv, self.G,
                                ssm_view.pool, ssm_view.state_in, ssm_view.state_out, batch.seg_offsets, segments,
-                               decay_t=decay, kscale_t=dt, skip_h=self.skip)
+                               decay_t=decay, kscale_t=dt, skip_h=self.skip, max_len=batch.max_q_len)
         y = kernels.group_norm_gate(y, self.norm_w, self.eps, self.norm_groups, gate=u[:, :inner], gate_act="silu",
                                     gate_before=True, out_dtype=self.dtype)
         return self.o_proj.forward(y)

@@ -39,13 +39,18 @@ def _close(got, want, tol, what):
     assert err < tol, f"{what}: error {err:.3e}"
 
 
+@pytest.mark.parametrize("piece", [0, 4, 7])
 @pytest.mark.parametrize("heads,groups,dk,dv", [(2, 2, 16, 24), (4, 2, 48, 8), (3, 1, 5, 3), (2, 2, 128, 64), (1, 1, 200, 40)])
-def test_decay_scan_segments_and_states(heads, groups, dk, dv):
+def test_decay_scan_segments_and_states(heads, groups, dk, dv, piece, monkeypatch):
     """Three segments of unequal length in one launch, one from a zero state, two from states that an earlier launch
-    left (rows used again); decays per token, a scale on k, a skip term; against the recurrence written out."""
+    left (rows used again); decays per token, a scale on k, a skip term; against the recurrence written out.  In one
+    pass (`piece` 0) and with the segments cut into pieces of 4 and of 7 tokens that run side by side (segments shorter
+    than a piece, of exactly some pieces, and with a rest)."""
     from infinilm_amd import kernels
+    monkeypatch.setattr(kernels, "SCAN_PIECE", piece)
+    monkeypatch.setattr(kernels, "SCAN_PIECE_FROM", 1)
     g = torch.Generator().manual_seed(heads * 100 + dk)
-    lens_a, lens_b = [7, 1, 19], [5, 33, 2]
+    lens_a, lens_b = [7, 1, 19], [8, 33, 2]
     pool = torch.zeros((6, heads, dv, dk), device=DEV)
     want, data = {}, {}
     skip = torch.randn(heads, generator=g)
@@ -66,7 +71,7 @@ def test_decay_scan_segments_and_states(heads, groups, dk, dv):
         sin = torch.tensor([0, 0, 0] if phase == 0 else rows, dtype=torch.int32, device=DEV)
         sout = torch.tensor(rows, dtype=torch.int32, device=DEV)
         o = kernels.decay_scan(q, k, v, heads, dk, dv, groups, pool, sin, sout, offs, 3, decay_t=cat(3).contiguous(),
-                               kscale_t=cat(4).contiguous(), skip_h=skip.to(DEV))
+                               kscale_t=cat(4).contiguous(), skip_h=skip.to(DEV), max_len=max(lens))
         at = 0
         for r, (a, b) in enumerate(cut):
             _close(o[at:at + b - a].cpu().view(-1, heads, dv), want[r][a:b], 2e-5, f"segment {r} phase {phase}")
@@ -88,7 +93,7 @@ def test_decay_scan_far_key_stands_out():
     pool = torch.zeros((2, 1, dv, dk), device=DEV)
     one = torch.tensor([1], dtype=torch.int32, device=DEV)
     o = kernels.decay_scan(q.to(DEV), k.to(DEV), v.to(DEV), 1, dk, dv, 1, pool, torch.zeros(1, dtype=torch.int32, device=DEV), one,
-                           torch.tensor([0, n], dtype=torch.int32, device=DEV), 1, decay_h=decay.to(DEV))
+                           torch.tensor([0, n], dtype=torch.int32, device=DEV), 1, decay_h=decay.to(DEV), max_len=n)
     _close(o.cpu(), want, 2e-5, "far key")
     assert float((want[-1] - 100 * decay.double() ** (n - 4) * v[3].double()).abs().max()) < 0.2 * float(want[-1].abs().max())
 
@@ -112,7 +117,8 @@ def test_causal_conv_carries_its_last_inputs(taps):
         x = torch.cat([xs[r][a:c] for r, (a, c) in enumerate(cut)]).to(DEV)
         offs = torch.tensor([0, lens[0], lens[0] + lens[1], sum(lens)], dtype=torch.int32, device=DEV)
         sin = torch.zeros(3, dtype=torch.int32, device=DEV) if phase == 0 else rows
-        y = kernels.causal_conv(x, w.to(DEV), b.to(DEV), pool, sin, rows, offs, 3, "silu")
+        seg = torch.tensor([r for r, n in enumerate(lens) for _ in range(n)], dtype=torch.int32, device=DEV)
+        y = kernels.causal_conv(x, w.to(DEV), b.to(DEV), pool, sin, rows, seg, offs, 3, "silu")
         at = 0
         for r, (a, c) in enumerate(cut):
             _close(y[at:at + c - a].cpu(), want[r][a:c], 1e-5, f"taps {taps} segment {r} phase {phase}")
