@@ -58,6 +58,7 @@ _SIGNATURES = {
     "ilm_ssm_steps": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "ilm_unit_qk_kvwrite": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P],
     "ilm_weighted_sum": [_P, _P, _P, _L, _F, _F, _I, _I, _I, _P],
+    "ilm_norm_add_norm": [_P, _P, _P, _P, _P, _I, _I, _F, _F, _F, _I, _I, _I, _I, _P],
 }
 
 

@@ -541,6 +541,40 @@ extern "C" int ilm_group_norm_gate(void* out, const void* x, const void* gate, c
 }
 
 // ------------------------------------------------------------------------------------------
+// A branch's output normed, added to the residual stream, and the stream normed for the next sublayer, in one pass:
+//   r += alpha * (y / sqrt(mean(y^2) + eps_b) * wb);   x = r / sqrt(mean(r^2) + eps) * w
+// One block a row; r is float, y and x have their own types.  Sums in an order that depends on the width only.
+// ------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+norm_add_norm_kernel(void* __restrict__ x, float* __restrict__ r, const void* __restrict__ y, const void* __restrict__ wb,
+                     const void* __restrict__ w, int H, float alpha, float eps_b, float eps, int x_dt, int y_dt, int wb_dt, int w_dt) {
+    __shared__ float red[4];
+    const size_t base = (size_t)blockIdx.x * H;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < H; j += 256) {
+        const float v = ldf(y, y_dt, base + j);
+        ss = fmaf(v, v, ss);
+    }
+    const float rb = alpha / sqrtf(block_sum<4>(ss, red) / (float)H + eps_b);
+    ss = 0.f;
+    for (int j = threadIdx.x; j < H; j += 256) {
+        const float v = fmaf(ldf(y, y_dt, base + j) * rb, ldf(wb, wb_dt, j), r[base + j]);
+        r[base + j] = v;
+        ss = fmaf(v, v, ss);
+    }
+    const float rs = 1.0f / sqrtf(block_sum<4>(ss, red) / (float)H + eps);
+    for (int j = threadIdx.x; j < H; j += 256) stf(x, x_dt, base + j, r[base + j] * rs * ldf(w, w_dt, j));
+}
+
+extern "C" int ilm_norm_add_norm(void* x, void* r, const void* y, const void* wb, const void* w, int rows, int H, float alpha,
+                                 float eps_b, float eps, int x_dt, int y_dt, int wb_dt, int w_dt, hipStream_t stream) {
+    ILM_REQUIRE(rows > 0 && H > 0, "norm_add_norm: bad sizes");
+    norm_add_norm_kernel<<<rows, 256, 0, stream>>>(x, (float*)r, y, wb, w, H, alpha, eps_b, eps, x_dt, y_dt, wb_dt, w_dt);
+    ILM_LAUNCH_CHECK("norm_add_norm");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
 // Short causal convolution over the tokens of each request, per channel, with bias and activation:
 //   y[t, c] = act(b[c] + sum_i w[c, i] * x[t - (taps - 1) + i, c]),   the last tap is the token's own input.
 // Inputs before a request's first token of this step come from its state row (the last taps - 1 inputs of the

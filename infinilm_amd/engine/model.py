@@ -99,6 +99,7 @@ class CausalLM:
             view = cache.view(run.cache, batch, run.writes_cache) if run.cache is not None else None
             self.blocks[run.layer].forward(stream, batch, view)
             if taps is not None:
+                stream.settle()
                 taps[f"run{i}"] = (stream.residual.clone(), None if stream.pending is None else stream.pending.clone(),
                                    stream.pending_scale)
         if batch.num_wanted == 0:
@@ -112,6 +113,7 @@ class CausalLM:
                 else:
                     pend = kernels.gather_rows(pend, batch.want_rows)
                 last.push(pend, stream.pending_scale)
+                last.pending_norm = stream.pending_norm     # a norm still due to the branch works row by row
             stream = last
         x = self.final_norm.forward(stream)
         return self.output_head.forward(x)

@@ -1215,3 +1215,23 @@ def weighted_sum(x: torch.Tensor, y: torch.Tensor, a: float, b: float, out_dtype
     _run("ilm_weighted_sum", out.data_ptr(), x.data_ptr(), y.data_ptr(), x.numel(), float(a), float(b), _dt(out), _dt(x),
          _dt(y), _stream())
     return out
+
+
+def norm_add_norm(residual: torch.Tensor, branch: torch.Tensor, branch_weight: torch.Tensor, branch_eps: float, alpha: float,
+                  weight: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """residual += alpha * rmsnorm(branch) * branch_weight (in place, float32), then the residual's own RMS norm times
+    `weight` as out_dtype: a branch that is normed before it joins the stream, and the norm before the next sublayer,
+    in one kernel."""
+    _dev(residual, branch, branch_weight, weight)
+    rows, H = residual.shape
+    if residual.dtype != F32 or not residual.is_contiguous():
+        raise KernelError("the residual stream is a contiguous float32 tensor")
+    if tuple(branch.shape) != (rows, H) or not branch.is_contiguous():
+        raise KernelError(f"branch {tuple(branch.shape)} does not match residual {tuple(residual.shape)}")
+    for wt in (branch_weight, weight):
+        if wt.shape != (H,) or not wt.is_contiguous():
+            raise KernelError(f"norm weight has shape {tuple(wt.shape)}, expected ({H},)")
+    out = torch.empty((rows, H), dtype=out_dtype, device=residual.device)
+    _run("ilm_norm_add_norm", out.data_ptr(), residual.data_ptr(), branch.data_ptr(), branch_weight.data_ptr(), weight.data_ptr(),
+         rows, H, float(alpha), float(branch_eps), float(eps), _dt(out), _dt(branch), _dt(branch_weight), _dt(weight), _stream())
+    return out

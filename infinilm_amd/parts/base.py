@@ -78,12 +78,26 @@ class ResidualStream:
         self.residual = residual
         self.pending: Optional[torch.Tensor] = None
         self.pending_scale: float = 1.0
+        # a branch that is still to be normed by `pending_norm` before it is added (an arrangement with a norm on every
+        # sublayer's output): a norm that knows how does both in its own kernel, anybody else calls `settle()` first
+        self.pending_norm = None
 
     def push(self, branch: torch.Tensor, scale: float) -> None:
         if self.pending is not None:
             raise RuntimeError("a branch is already pending; a norm must fold it first")
         self.pending = branch
         self.pending_scale = scale
+
+    def push_normed(self, branch: torch.Tensor, norm, scale: float) -> None:
+        """`branch` [T, hidden] joins the stream as norm(branch) * scale; the norm is applied when the stream is next read."""
+        self.push(branch, scale)
+        self.pending_norm = norm
+
+    def settle(self) -> None:
+        """Applies a norm that is still due to the pending branch, so that `pending` is what is added."""
+        if self.pending_norm is not None:
+            norm, self.pending_norm = self.pending_norm, None
+            self.pending = norm.apply(self.pending)
 
 
 @dataclass

@@ -68,8 +68,9 @@ class PreNormBlock:
 @register_arrangement("sandwich_norm")
 class SandwichNormBlock:
     """x += s * norm1b(mixer(norm1(x))); x += s * norm2b(ffn(norm2(x))): a norm before every sublayer and another on
-    its output before the sum.  A layer may have no feed-forward (no `ffn`, `norm2`, `norm2b` among its parts).  The
-    norms on the outputs give float32 rows, which the next norm's kernel adds to the float32 residual stream."""
+    its output before the sum.  A layer may have no feed-forward (no `ffn`, `norm2`, `norm2b` among its parts).  A
+    sublayer's output is left with the stream together with its norm (`ResidualStream.push_normed`): the next norm's
+    kernel norms it, adds it to the float32 residual stream and norms the stream, in one pass."""
 
     def __init__(self, spec: LayerSpec, ctx: BuildContext):
         self.spec = spec
@@ -104,10 +105,10 @@ class SandwichNormBlock:
 
     def forward(self, stream: ResidualStream, batch, cache_view) -> None:
         y = self.mixer.forward(self.norm1.forward(stream), batch, cache_view)
-        stream.push(self.norm1b.apply(y), self.residual_scale)
+        stream.push_normed(y, self.norm1b, self.residual_scale)      # (normed and added inside the next norm's kernel)
         if self.ffn is not None:
             y = self.ffn.forward(self.norm2.forward(stream), batch)
-            stream.push(self.norm2b.apply(y), self.residual_scale)
+            stream.push_normed(y, self.norm2b, self.residual_scale)
 
 
 def build_block(spec: LayerSpec, ctx: BuildContext):

@@ -39,12 +39,21 @@ class RMSNorm(Norm):
         return kernels.group_norm_gate(x, self.weight, self.eps, 1, out_dtype=out_dtype)
 
     def tail(self, stream: ResidualStream, scale: float, rows: int):
+        stream.settle()
         if stream.pending is not None or self.dtype != torch.bfloat16 or rows > kernels.TAIL_MAX_ROWS:
             return None
         return NormTail(stream.residual, float(scale), self.weight, self.eps)
 
     def forward(self, stream: ResidualStream, frag: bool = False):
         """`frag`: the consumer takes its rows in fragment order (`kernels.FragRows`)."""
+        post = stream.pending_norm
+        if post is not None and not frag and isinstance(post, RMSNorm) and stream.pending.dim() == 2:
+            # the branch's own norm, the sum and this norm in one kernel
+            x = kernels.norm_add_norm(stream.residual, stream.pending, post.weight, post.eps, stream.pending_scale, self.weight,
+                                      self.eps, self.dtype)
+            stream.pending, stream.pending_scale, stream.pending_norm = None, 1.0, None
+            return x
+        stream.settle()
         x = kernels.add_rmsnorm(stream.residual, stream.pending, self.weight, stream.pending_scale, self.eps,
                                 self.dtype, frag=frag)
         stream.pending = None
