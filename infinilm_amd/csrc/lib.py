@@ -53,12 +53,12 @@ _SIGNATURES = {
     "ilm_unary": [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "ilm_lin_prep": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "ilm_decay_scan": [_P, _I, _P, _P, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P],
-    "ilm_group_norm_gate": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _I, _P],
+    "ilm_group_norm_gate": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _I, _I, _L, _P],
     "ilm_causal_conv": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "ilm_ssm_steps": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "ilm_unit_qk_kvwrite": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P],
     "ilm_weighted_sum": [_P, _P, _P, _L, _F, _F, _I, _I, _I, _P],
-    "ilm_norm_add_norm": [_P, _P, _P, _P, _P, _I, _I, _F, _F, _F, _I, _I, _I, _I, _P],
+    "ilm_norm_add_norm": [_P, _P, _P, _P, _P, _I, _I, _F, _F, _F, _I, _I, _I, _I, _I, _L, _P],
 }
 
 

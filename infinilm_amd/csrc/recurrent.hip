@@ -156,6 +156,19 @@ extern "C" int ilm_lin_prep(void* out, const void* in, const void* pos, const vo
 // floor(first row of r / piece) + r + p: slots of different segments never meet, and floor(T / piece) + R slots hold all.
 // A block finds its (segment, piece) from its slot by bisection over the segments' first slots.
 // ------------------------------------------------------------------------------------------
+// Sums over the KP lanes of a column group, for the four columns a thread holds: two exchanges halve the columns a lane
+// goes on with (lanes with bit 0 clear keep columns 0 and 1, then bit 1 picks one of the two), the remaining steps fold
+// one number.  At the end lane kp (kp < 4) of the group holds the sum of column 2 * (kp & 1) + ((kp >> 1) & 1): five
+// exchanges for 16 lanes where four separate folds take sixteen.  KP >= 4.
+__device__ __forceinline__ float sc_fold4(const float (&acc)[4], int kp, int KP) {
+    const bool b0 = kp & 1, b1 = kp & 2;
+    const float s0 = __shfl_xor(b0 ? acc[0] : acc[2], 1, 64), s1 = __shfl_xor(b0 ? acc[1] : acc[3], 1, 64);
+    const float k0 = (b0 ? acc[2] : acc[0]) + s0, k1 = (b0 ? acc[3] : acc[1]) + s1;
+    float v = (b1 ? k1 : k0) + __shfl_xor(b1 ? k0 : k1, 2, 64);
+    for (int off = 4; off < KP; off <<= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
 #define SC_NK 8
 #define SC_WHOLE 0
 #define SC_LOCAL 1
@@ -254,10 +267,18 @@ decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__
         if (MODE == SC_LOCAL) {
             aprod *= a;
         } else {
+            if (VC == 4 && KP >= 4) {
+                const float (&a4)[4] = reinterpret_cast<const float (&)[4]>(acc);
+                const float tot = sc_fold4(a4, kp, KP);
+                const int c = 2 * (kp & 1) + ((kp >> 1) & 1);
+                const float vsel = c == 0 ? vcur[0] : c == 1 ? vcur[VC > 1 ? 1 : 0] : c == 2 ? vcur[VC > 2 ? 2 : 0] : vcur[VC > 3 ? 3 : 0];
+                if (kp < 4 && vc0 + c < dv) o[(size_t)t * o_stride + (size_t)h * dv + vc0 + c] = fmaf(skip, vsel, tot);
+            } else {
 #pragma unroll
-            for (int c = 0; c < VC; ++c) {
-                for (int off = 1; off < KP; off <<= 1) acc[c] += __shfl_xor(acc[c], off, 64);
-                if (kp == 0 && vc0 + c < dv) o[(size_t)t * o_stride + (size_t)h * dv + vc0 + c] = fmaf(skip, vcur[c], acc[c]);
+                for (int c = 0; c < VC; ++c) {
+                    for (int off = 1; off < KP; off <<= 1) acc[c] += __shfl_xor(acc[c], off, 64);
+                    if (kp == 0 && vc0 + c < dv) o[(size_t)t * o_stride + (size_t)h * dv + vc0 + c] = fmaf(skip, vcur[c], acc[c]);
+                }
             }
         }
     }
@@ -383,11 +404,20 @@ decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __rest
             if (MODE == SC_LOCAL) {
                 aprod *= a;
             } else {
+                if (VC == 4 && KP >= 4) {
+                    const float (&a4)[4] = reinterpret_cast<const float (&)[4]>(acc);
+                    const float tot = sc_fold4(a4, kp, KP);
+                    const int c = 2 * (kp & 1) + ((kp >> 1) & 1);
+                    const float vsel = c == 0 ? vcur[0] : c == 1 ? vcur[VC > 1 ? 1 : 0] : c == 2 ? vcur[VC > 2 ? 2 : 0] : vcur[VC > 3 ? 3 : 0];
+                    if (kp < 4 && vb + cl + c < dv)
+                        o[(size_t)(tb + tt) * o_stride + (size_t)h * dv + vb + cl + c] = fmaf(skip, vsel, tot);
+                } else {
 #pragma unroll
-                for (int c = 0; c < VC; ++c) {
-                    for (int off = 1; off < KP; off <<= 1) acc[c] += __shfl_xor(acc[c], off, 64);
-                    if (kp == 0 && vb + cl + c < dv)
-                        o[(size_t)(tb + tt) * o_stride + (size_t)h * dv + vb + cl + c] = fmaf(skip, vcur[c], acc[c]);
+                    for (int c = 0; c < VC; ++c) {
+                        for (int off = 1; off < KP; off <<= 1) acc[c] += __shfl_xor(acc[c], off, 64);
+                        if (kp == 0 && vb + cl + c < dv)
+                            o[(size_t)(tb + tt) * o_stride + (size_t)h * dv + vb + cl + c] = fmaf(skip, vcur[c], acc[c]);
+                    }
                 }
             }
         }
@@ -496,7 +526,8 @@ template <int LANES>   // threads an item: 64 (four items a block) or 256
 __global__ void __launch_bounds__(256)
 group_norm_gate_kernel(void* __restrict__ out, const void* __restrict__ x, const void* __restrict__ gate,
                        const void* __restrict__ w, int rows, int n, int groups, int x_stride, int gate_stride,
-                       int out_stride, float eps, int gate_act, int gate_before, int out_dt, int x_dt, int gate_dt, int w_dt) {
+                       int out_stride, float eps, int gate_act, int gate_before, int out_dt, int x_dt, int gate_dt, int w_dt,
+                       int parts, size_t pstride) {
     __shared__ float red[4];
     const int item = LANES == 64 ? blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
     const int lane = LANES == 64 ? (threadIdx.x & 63) : threadIdx.x;
@@ -508,6 +539,7 @@ group_norm_gate_kernel(void* __restrict__ out, const void* __restrict__ x, const
     float ss = 0.f;
     for (int j = lane; j < gs; j += LANES) {
         float y = ldf(x, x_dt, xb + j);
+        for (int p = 1; p < parts; ++p) y += ldf(x, x_dt, p * pstride + xb + j);
         if (pre) y *= act_f(ldf(gate, gate_dt, gb + j), gate_act);
         ss = fmaf(y, y, ss);
     }
@@ -515,6 +547,7 @@ group_norm_gate_kernel(void* __restrict__ out, const void* __restrict__ x, const
     const float rstd = 1.0f / sqrtf(ss / (float)gs + eps);
     for (int j = lane; j < gs; j += LANES) {
         float y = ldf(x, x_dt, xb + j);
+        for (int p = 1; p < parts; ++p) y += ldf(x, x_dt, p * pstride + xb + j);
         if (pre) y *= act_f(ldf(gate, gate_dt, gb + j), gate_act);
         y *= rstd;
         if (w != nullptr) y *= ldf(w, w_dt, (size_t)g * gs + j);
@@ -525,16 +558,17 @@ group_norm_gate_kernel(void* __restrict__ out, const void* __restrict__ x, const
 
 extern "C" int ilm_group_norm_gate(void* out, const void* x, const void* gate, const void* w, int rows, int n, int groups,
                                    int x_stride, int gate_stride, int out_stride, float eps, int gate_act, int gate_before,
-                                   int out_dt, int x_dt, int gate_dt, int w_dt, hipStream_t stream) {
+                                   int out_dt, int x_dt, int gate_dt, int w_dt, int parts, long pstride, hipStream_t stream) {
+    ILM_REQUIRE(parts >= 1, "group_norm_gate: %d parts", parts);
     ILM_REQUIRE(rows > 0 && n > 0 && groups > 0 && n % groups == 0, "group_norm_gate: %d elements do not divide into %d groups", n, groups);
     ILM_REQUIRE((long)rows * groups < (1L << 31) - 4, "group_norm_gate: too many rows");
     if (n / groups > 512) {
         group_norm_gate_kernel<256><<<rows * groups, 256, 0, stream>>>(out, x, gate, w, rows, n, groups, x_stride, gate_stride,
-                                                                       out_stride, eps, gate_act, gate_before, out_dt, x_dt, gate_dt, w_dt);
+                                                                       out_stride, eps, gate_act, gate_before, out_dt, x_dt, gate_dt, w_dt, parts, (size_t)pstride);
     } else {
         const int blocks = (int)(((long)rows * groups + 3) / 4);
         group_norm_gate_kernel<64><<<blocks, 256, 0, stream>>>(out, x, gate, w, rows, n, groups, x_stride, gate_stride, out_stride,
-                                                               eps, gate_act, gate_before, out_dt, x_dt, gate_dt, w_dt);
+                                                               eps, gate_act, gate_before, out_dt, x_dt, gate_dt, w_dt, parts, (size_t)pstride);
     }
     ILM_LAUNCH_CHECK("group_norm_gate");
     return 0;
@@ -547,18 +581,22 @@ extern "C" int ilm_group_norm_gate(void* out, const void* x, const void* gate, c
 // ------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)
 norm_add_norm_kernel(void* __restrict__ x, float* __restrict__ r, const void* __restrict__ y, const void* __restrict__ wb,
-                     const void* __restrict__ w, int H, float alpha, float eps_b, float eps, int x_dt, int y_dt, int wb_dt, int w_dt) {
+                     const void* __restrict__ w, int H, float alpha, float eps_b, float eps, int x_dt, int y_dt, int wb_dt, int w_dt,
+                     int parts, size_t pstride) {
     __shared__ float red[4];
     const size_t base = (size_t)blockIdx.x * H;
     float ss = 0.f;
     for (int j = threadIdx.x; j < H; j += 256) {
-        const float v = ldf(y, y_dt, base + j);
+        float v = ldf(y, y_dt, base + j);
+        for (int p = 1; p < parts; ++p) v += ldf(y, y_dt, p * pstride + base + j);
         ss = fmaf(v, v, ss);
     }
     const float rb = alpha / sqrtf(block_sum<4>(ss, red) / (float)H + eps_b);
     ss = 0.f;
     for (int j = threadIdx.x; j < H; j += 256) {
-        const float v = fmaf(ldf(y, y_dt, base + j) * rb, ldf(wb, wb_dt, j), r[base + j]);
+        float yv = ldf(y, y_dt, base + j);
+        for (int p = 1; p < parts; ++p) yv += ldf(y, y_dt, p * pstride + base + j);
+        const float v = fmaf(yv * rb, ldf(wb, wb_dt, j), r[base + j]);
         r[base + j] = v;
         ss = fmaf(v, v, ss);
     }
@@ -566,10 +604,103 @@ norm_add_norm_kernel(void* __restrict__ x, float* __restrict__ r, const void* __
     for (int j = threadIdx.x; j < H; j += 256) stf(x, x_dt, base + j, r[base + j] * rs * ldf(w, w_dt, j));
 }
 
+// eight consecutive elements as floats / from floats (16-byte accesses for bfloat16, two for float)
+__device__ __forceinline__ void ld8(const void* p, int dt, size_t i, float (&v)[8]) {
+    if (dt == ILM_DTYPE_F32) {
+        const float4 a = *reinterpret_cast<const float4*>((const float*)p + i), b = *reinterpret_cast<const float4*>((const float*)p + i + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        uint16_t t[8];
+        *reinterpret_cast<uint4*>(t) = *reinterpret_cast<const uint4*>((const uint16_t*)p + i);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = bf16_bits_to_f32(t[e]);
+    }
+}
+__device__ __forceinline__ void st8(void* p, int dt, size_t i, const float (&v)[8]) {
+    if (dt == ILM_DTYPE_F32) {
+        *reinterpret_cast<float4*>((float*)p + i) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4*>((float*)p + i + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+        uint16_t t[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[e] = __builtin_bit_cast(uint16_t, (__bf16)v[e]);
+        *reinterpret_cast<uint4*>((uint16_t*)p + i) = *reinterpret_cast<uint4*>(t);
+    }
+}
+
+// The same for widths that are multiples of 8 up to 8 * 256 * NITER: a thread keeps its pieces of the row in registers
+// from the first sum to the last store, so y is read once, r read and written once, x written once.
+template <int NITER>
+__global__ void __launch_bounds__(256)
+norm_add_norm_vec_kernel(void* __restrict__ x, float* __restrict__ r, const void* __restrict__ y, const void* __restrict__ wb,
+                         const void* __restrict__ w, int H, float alpha, float eps_b, float eps, int x_dt, int y_dt, int wb_dt, int w_dt,
+                         int parts, size_t pstride) {
+    __shared__ float red[4];
+    const size_t base = (size_t)blockIdx.x * H;
+    float v[NITER][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < NITER; ++it) {
+        const int j = (it * 256 + threadIdx.x) * 8;
+        if (j < H) {
+            ld8(y, y_dt, base + j, v[it]);
+            for (int p = 1; p < parts; ++p) {      // the parts of a product that was split over K, summed in order
+                float more[8];
+                ld8(y, y_dt, p * pstride + base + j, more);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[it][e] += more[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss = fmaf(v[it][e], v[it][e], ss);
+        }
+    }
+    const float rb = alpha / sqrtf(block_sum<4>(ss, red) / (float)H + eps_b);
+    ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < NITER; ++it) {
+        const int j = (it * 256 + threadIdx.x) * 8;
+        if (j < H) {
+            float g[8], q[8];
+            ld8(wb, wb_dt, j, g);
+            ld8(r, ILM_DTYPE_F32, base + j, q);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                v[it][e] = fmaf(v[it][e] * rb, g[e], q[e]);
+                ss = fmaf(v[it][e], v[it][e], ss);
+            }
+            st8(r, ILM_DTYPE_F32, base + j, v[it]);
+        }
+    }
+    const float rs = 1.0f / sqrtf(block_sum<4>(ss, red) / (float)H + eps);
+#pragma unroll
+    for (int it = 0; it < NITER; ++it) {
+        const int j = (it * 256 + threadIdx.x) * 8;
+        if (j < H) {
+            float g[8], out[8];
+            ld8(w, w_dt, j, g);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) out[e] = v[it][e] * rs * g[e];
+            st8(x, x_dt, base + j, out);
+        }
+    }
+}
+
 extern "C" int ilm_norm_add_norm(void* x, void* r, const void* y, const void* wb, const void* w, int rows, int H, float alpha,
-                                 float eps_b, float eps, int x_dt, int y_dt, int wb_dt, int w_dt, hipStream_t stream) {
-    ILM_REQUIRE(rows > 0 && H > 0, "norm_add_norm: bad sizes");
-    norm_add_norm_kernel<<<rows, 256, 0, stream>>>(x, (float*)r, y, wb, w, H, alpha, eps_b, eps, x_dt, y_dt, wb_dt, w_dt);
+                                 float eps_b, float eps, int x_dt, int y_dt, int wb_dt, int w_dt, int parts, long pstride,
+                                 hipStream_t stream) {
+    ILM_REQUIRE(rows > 0 && H > 0 && parts >= 1, "norm_add_norm: bad sizes");
+    const bool al = pstride % 8 == 0 && (((uintptr_t)x | (uintptr_t)r | (uintptr_t)y | (uintptr_t)wb | (uintptr_t)w) & 15) == 0;
+    if (al && H % 8 == 0 && H <= 8192) {
+#define NAN_ARGS x, (float*)r, y, wb, w, H, alpha, eps_b, eps, x_dt, y_dt, wb_dt, w_dt, parts, (size_t)pstride
+        if (H <= 2048) norm_add_norm_vec_kernel<1><<<rows, 256, 0, stream>>>(NAN_ARGS);
+        else if (H <= 4096) norm_add_norm_vec_kernel<2><<<rows, 256, 0, stream>>>(NAN_ARGS);
+        else norm_add_norm_vec_kernel<4><<<rows, 256, 0, stream>>>(NAN_ARGS);
+#undef NAN_ARGS
+        ILM_LAUNCH_CHECK("norm_add_norm");
+        return 0;
+    }
+    norm_add_norm_kernel<<<rows, 256, 0, stream>>>(x, (float*)r, y, wb, w, H, alpha, eps_b, eps, x_dt, y_dt, wb_dt, w_dt, parts,
+                                                   (size_t)pstride);
     ILM_LAUNCH_CHECK("norm_add_norm");
     return 0;
 }

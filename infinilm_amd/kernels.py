@@ -1119,8 +1119,14 @@ def group_norm_gate(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
                     gate: Optional[torch.Tensor] = None, gate_act: str = "none", gate_before: bool = False,
                     out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
     """RMS norm of every row in `groups` equal parts (each by its own root mean square, eps inside the root), times
-    `weight` [n] if given; `gate` [T, n]: times act(gate), before the norm or after it.  Sums in float32."""
+    `weight` [n] if given; `gate` [T, n]: times act(gate), before the norm or after it.  Sums in float32.
+    x may come as contiguous parts [P, T, n] that are summed first (a product that was split over K)."""
     _dev(x, weight, gate)
+    parts, pstride = 1, 0
+    if x.dim() == 3:
+        if not x.is_contiguous():
+            raise KernelError("parts must be contiguous")
+        parts, pstride, x = x.shape[0], x.stride(0), x[0]
     _rows(x, "x")
     T, n = x.shape
     if groups <= 0 or n % groups:
@@ -1134,7 +1140,8 @@ def group_norm_gate(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
     out = torch.empty((T, n), dtype=out_dtype or x.dtype, device=x.device)
     _run("ilm_group_norm_gate", out.data_ptr(), x.data_ptr(), _ptr(gate), _ptr(weight), T, n, int(groups), x.stride(0),
          gate.stride(0) if gate is not None else 0, out.stride(0), float(eps), _act(gate_act), int(bool(gate_before)),
-         _dt(out), _dt(x), _dt(gate) if gate is not None else 0, _dt(weight) if weight is not None else 0, _stream())
+         _dt(out), _dt(x), _dt(gate) if gate is not None else 0, _dt(weight) if weight is not None else 0, parts, pstride,
+         _stream())
     return out
 
 
@@ -1221,17 +1228,21 @@ def norm_add_norm(residual: torch.Tensor, branch: torch.Tensor, branch_weight: t
                   weight: torch.Tensor, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
     """residual += alpha * rmsnorm(branch) * branch_weight (in place, float32), then the residual's own RMS norm times
     `weight` as out_dtype: a branch that is normed before it joins the stream, and the norm before the next sublayer,
-    in one kernel."""
+    in one kernel.  `branch` is [rows, H] or float32 parts [P, rows, H] that are summed first."""
     _dev(residual, branch, branch_weight, weight)
     rows, H = residual.shape
     if residual.dtype != F32 or not residual.is_contiguous():
         raise KernelError("the residual stream is a contiguous float32 tensor")
-    if tuple(branch.shape) != (rows, H) or not branch.is_contiguous():
+    parts, pstride = 1, 0
+    if branch.dim() == 3:      # float32 parts of a product that was split over K
+        parts, pstride = branch.shape[0], branch.stride(0)
+    if tuple(branch.shape[-2:]) != (rows, H) or not branch.is_contiguous():
         raise KernelError(f"branch {tuple(branch.shape)} does not match residual {tuple(residual.shape)}")
     for wt in (branch_weight, weight):
         if wt.shape != (H,) or not wt.is_contiguous():
             raise KernelError(f"norm weight has shape {tuple(wt.shape)}, expected ({H},)")
     out = torch.empty((rows, H), dtype=out_dtype, device=residual.device)
     _run("ilm_norm_add_norm", out.data_ptr(), residual.data_ptr(), branch.data_ptr(), branch_weight.data_ptr(), weight.data_ptr(),
-         rows, H, float(alpha), float(branch_eps), float(eps), _dt(out), _dt(branch), _dt(branch_weight), _dt(weight), _stream())
+         rows, H, float(alpha), float(branch_eps), float(eps), _dt(out), _dt(branch), _dt(branch_weight), _dt(weight), parts, pstride,
+         _stream())
     return out

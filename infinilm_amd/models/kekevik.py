@@ -156,8 +156,7 @@ def build_spec(cfg: KekevikConfig) -> ModelSpec:
         if layer.ff is not None:
             parts.update(norm2=norm, norm2b=norm,
                          ffn=PartSpec("activation_mlp", {"hidden_size": W, "intermediate_size": layer.ff, "activation": "relu2",
-                                                         "bias": False, "names": ("up", "down"), "suffix": "",
-                                                         "whole_output": True}))
+                                                         "bias": False, "names": ("up", "down"), "suffix": ""}))
             names.update(norm2="norm2", ffn="mlp", norm2b="norm2b")
         layers.append(LayerSpec(prefix=f"l{i}", arrangement="sandwich_norm", parts=parts, names=names))
     order = [LayerRun(layer=i, cache=i, writes_cache=True) for i in range(len(layers))]

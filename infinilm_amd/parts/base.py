@@ -89,7 +89,8 @@ class ResidualStream:
         self.pending_scale = scale
 
     def push_normed(self, branch: torch.Tensor, norm, scale: float) -> None:
-        """`branch` [T, hidden] joins the stream as norm(branch) * scale; the norm is applied when the stream is next read."""
+        """`branch` ([T, hidden], or float32 parts [P, T, hidden] of a product split over K) joins the stream as
+        norm(branch) * scale; the norm is applied when the stream is next read."""
         self.push(branch, scale)
         self.pending_norm = norm
 

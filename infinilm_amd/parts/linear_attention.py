@@ -30,7 +30,7 @@ class DecayLinearAttention(Mixer):
     def __init__(self, hidden_size: int, heads: int, key_dim: int, value_dim: int, decay: Sequence[float], eps: float,
                  ctx: BuildContext, activation: str = "none", rotary: Optional[dict] = None, k_scale: float = 1.0,
                  norm: str = "head", norm_weight: bool = False, gate_act: str = "silu",
-                 names: Sequence[str] = ("q", "k", "v", "g", "o", "norm"), suffix: str = ""):
+                 names: Sequence[str] = ("q", "k", "v", "g", "o", "norm"), suffix: str = "", whole_output: bool = False):
         self.H, self.dk, self.dv = int(heads), int(key_dim), int(value_dim)
         if len(decay) != self.H:
             raise ValueError(f"{len(decay)} decays for {self.H} heads")
@@ -41,6 +41,7 @@ class DecayLinearAttention(Mixer):
         self.activation, self.k_scale, self.eps = activation, float(k_scale), float(eps)
         self.norm_groups = self.H if norm == "head" else 1
         self.gate_act = gate_act
+        self.whole_output = bool(whole_output)    # never float32 parts still to be summed (see GQAttention)
         self.dtype = ctx.dtype
         kernels._act(activation), kernels._act(gate_act)
         qn, kn, vn, gn, on, self.norm_name = names
@@ -77,7 +78,7 @@ class DecayLinearAttention(Mixer):
                                max_len=batch.max_q_len)
         y = kernels.group_norm_gate(o, self.norm_w, self.eps, self.norm_groups, gate=rows[:, 2 * H * dk + H * dv:],
                                     gate_act=self.gate_act, out_dtype=self.dtype)
-        return self.o_proj.forward(y)
+        return self.o_proj.forward(y, allow_parts=not self.whole_output)
 
 
 @register_mixer("retention")

@@ -47,7 +47,7 @@ class RMSNorm(Norm):
     def forward(self, stream: ResidualStream, frag: bool = False):
         """`frag`: the consumer takes its rows in fragment order (`kernels.FragRows`)."""
         post = stream.pending_norm
-        if post is not None and not frag and isinstance(post, RMSNorm) and stream.pending.dim() == 2:
+        if post is not None and not frag and isinstance(post, RMSNorm):
             # the branch's own norm, the sum and this norm in one kernel
             x = kernels.norm_add_norm(stream.residual, stream.pending, post.weight, post.eps, stream.pending_scale, self.weight,
                                       self.eps, self.dtype)

@@ -72,8 +72,9 @@ def retention(h, W: Dict[str, torch.Tensor], m: dict, eps: float):
     k = proj(h, W["k"]).view(T, H, dk)
     v = proj(h, W["v"]).view(T, H, dv)
     rot = m.get("rot") or {"dims": 0, "base": 1.0}
-    q = torch.stack([rotate_half(q[t], t, rot["dims"], rot["base"]) for t in range(T)])
-    k = torch.stack([rotate_half(k[t], t, rot["dims"], rot["base"]) for t in range(T)]) * dk ** -0.5
+    dims, base = int(rot.get("dims", 0) or 0), float(rot.get("base", 1.0))
+    q = torch.stack([rotate_half(q[t], t, dims, base) for t in range(T)])
+    k = torch.stack([rotate_half(k[t], t, dims, base) for t in range(T)]) * dk ** -0.5
     o = decayed_outer_scan(q, k, v, torch.tensor(m["decay"], dtype=h.dtype))
     o = rms_unit(o, eps).reshape(T, H * dv) * silu(proj(h, W["g"]))
     return proj(o, W["o"])
