@@ -34,6 +34,30 @@ __device__ __forceinline__ float act_f(float x, int kind) {
     }
 }
 
+// eight consecutive elements as floats / from floats (16-byte accesses for bfloat16, two for float)
+__device__ __forceinline__ void ld8(const void* p, int dt, size_t i, float (&v)[8]) {
+    if (dt == ILM_DTYPE_F32) {
+        const float4 a = *reinterpret_cast<const float4*>((const float*)p + i), b = *reinterpret_cast<const float4*>((const float*)p + i + 4);
+        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    } else {
+        uint16_t t[8];
+        *reinterpret_cast<uint4*>(t) = *reinterpret_cast<const uint4*>((const uint16_t*)p + i);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = bf16_bits_to_f32(t[e]);
+    }
+}
+__device__ __forceinline__ void st8(void* p, int dt, size_t i, const float (&v)[8]) {
+    if (dt == ILM_DTYPE_F32) {
+        *reinterpret_cast<float4*>((float*)p + i) = make_float4(v[0], v[1], v[2], v[3]);
+        *reinterpret_cast<float4*>((float*)p + i + 4) = make_float4(v[4], v[5], v[6], v[7]);
+    } else {
+        uint16_t t[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) t[e] = __builtin_bit_cast(uint16_t, (__bf16)v[e]);
+        *reinterpret_cast<uint4*>((uint16_t*)p + i) = *reinterpret_cast<uint4*>(t);
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // out[t, j] = act(in[t, j]), rows of n elements with their own strides
 // ------------------------------------------------------------------------------------------
@@ -122,12 +146,68 @@ lin_prep_kernel(float* __restrict__ out, const void* __restrict__ in, const int*
     for (int j = 2 * nqk + threadIdx.x; j < n; j += 256) out[ob + j] = act_f(ldf(in, in_dt, ib + j), act);
 }
 
+// The same with eight elements a thread: head sizes and half the turned entries in multiples of 8, rows 16 bytes aligned.
+__global__ void __launch_bounds__(256)
+lin_prep_vec_kernel(float* __restrict__ out, const void* __restrict__ in, const int* __restrict__ pos,
+                    const float* __restrict__ freq, int heads, int dk, int dv, int rd, int in_stride, int act, float k_scale,
+                    int in_dt) {
+    const int t = blockIdx.x;
+    const int nqk = heads * dk, n = 2 * nqk + heads * dv;
+    const size_t ib = (size_t)t * in_stride, ob = (size_t)t * n;
+    const int half = rd >> 1, hp = half >> 3, rest = (dk - rd) >> 3;
+    const int per_head = hp + rest;                       // work items of a q or k head: turned pairs of pieces, then passing pieces
+    const int n_qk = 2 * heads * per_head, n_items = n_qk + (heads * dv >> 3);
+    const float p = rd > 0 ? (float)pos[t] : 0.f;
+    for (int it = threadIdx.x; it < n_items; it += 256) {
+        float a[8], o8[8];
+        if (it >= n_qk) {                                  // values
+            const size_t c = 2 * (size_t)nqk + (size_t)(it - n_qk) * 8;
+            ld8(in, in_dt, ib + c, a);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o8[e] = act_f(a[e], act);
+            st8(out, ILM_DTYPE_F32, ob + c, o8);
+            continue;
+        }
+        const int hs = it / per_head, piece = it % per_head;
+        const float sc = hs >= heads ? k_scale : 1.0f;
+        if (piece >= hp) {                                 // entries that pass
+            const size_t c = (size_t)hs * dk + rd + (size_t)(piece - hp) * 8;
+            ld8(in, in_dt, ib + c, a);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o8[e] = act_f(a[e], act) * sc;
+            st8(out, ILM_DTYPE_F32, ob + c, o8);
+            continue;
+        }
+        const int i0 = piece * 8;
+        const size_t c = (size_t)hs * dk + i0;
+        float b[8], o9[8];
+        ld8(in, in_dt, ib + c, a);
+        ld8(in, in_dt, ib + c + half, b);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float u = act_f(a[e], act), w = act_f(b[e], act);
+            float sn, cs;
+            sincosf(p * freq[i0 + e], &sn, &cs);
+            o8[e] = (u * cs - w * sn) * sc;
+            o9[e] = (w * cs + u * sn) * sc;
+        }
+        st8(out, ILM_DTYPE_F32, ob + c, o8);
+        st8(out, ILM_DTYPE_F32, ob + c + half, o9);
+    }
+}
+
 extern "C" int ilm_lin_prep(void* out, const void* in, const void* pos, const void* freq, int T_, int heads, int dk, int dv,
                             int rd, int in_stride, int act, float k_scale, int in_dt, hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && heads > 0 && dk > 0 && dv > 0, "lin_prep: bad sizes");
     ILM_REQUIRE(rd >= 0 && rd <= dk && rd % 2 == 0, "lin_prep: %d turned entries do not fit a head of %d", rd, dk);
     ILM_REQUIRE(rd == 0 || (freq != nullptr && pos != nullptr), "lin_prep: a rotation needs positions and frequencies");
     ILM_REQUIRE(in_stride >= 2 * heads * dk + heads * dv, "lin_prep: rows of %d elements are too short", in_stride);
+    if (dk % 8 == 0 && dv % 8 == 0 && rd % 16 == 0 && in_stride % 8 == 0 && (((uintptr_t)out | (uintptr_t)in) & 15) == 0) {
+        lin_prep_vec_kernel<<<T_, 256, 0, stream>>>((float*)out, in, (const int*)pos, (const float*)freq, heads, dk, dv, rd,
+                                                    in_stride, act, k_scale, in_dt);
+        ILM_LAUNCH_CHECK("lin_prep");
+        return 0;
+    }
     lin_prep_kernel<<<T_, 256, 0, stream>>>((float*)out, in, (const int*)pos, (const float*)freq, heads, dk, dv, rd, in_stride,
                                             act, k_scale, in_dt);
     ILM_LAUNCH_CHECK("lin_prep");
@@ -556,12 +636,91 @@ group_norm_gate_kernel(void* __restrict__ out, const void* __restrict__ x, const
     }
 }
 
+// The same with eight elements a thread and the group in registers between the sum and the stores: groups in multiples
+// of 8 up to 8 * LANES * NITER elements, rows 16 bytes aligned.
+template <int LANES, int NITER>
+__global__ void __launch_bounds__(256)
+group_norm_gate_vec_kernel(void* __restrict__ out, const void* __restrict__ x, const void* __restrict__ gate,
+                           const void* __restrict__ w, int rows, int n, int groups, int x_stride, int gate_stride,
+                           int out_stride, float eps, int gate_act, int gate_before, int out_dt, int x_dt, int gate_dt, int w_dt,
+                           int parts, size_t pstride) {
+    __shared__ float red[4];
+    const int item = LANES == 64 ? blockIdx.x * 4 + (threadIdx.x >> 6) : blockIdx.x;
+    const int lane = LANES == 64 ? (threadIdx.x & 63) : threadIdx.x;
+    if (item >= rows * groups) return;
+    const int t = item / groups, g = item % groups, gs = n / groups;
+    const size_t xb = (size_t)t * x_stride + (size_t)g * gs, gb = (size_t)t * gate_stride + (size_t)g * gs;
+    const size_t ob = (size_t)t * out_stride + (size_t)g * gs;
+    const bool pre = gate != nullptr && gate_before;
+    float v[NITER][8];
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < NITER; ++it) {
+        const int j = (it * LANES + lane) * 8;
+        if (j < gs) {
+            ld8(x, x_dt, xb + j, v[it]);
+            for (int p = 1; p < parts; ++p) {
+                float more[8];
+                ld8(x, x_dt, p * pstride + xb + j, more);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[it][e] += more[e];
+            }
+            if (pre) {
+                float gt[8];
+                ld8(gate, gate_dt, gb + j, gt);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[it][e] *= act_f(gt[e], gate_act);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) ss = fmaf(v[it][e], v[it][e], ss);
+        }
+    }
+    ss = LANES == 64 ? wave_sum(ss) : block_sum<4>(ss, red);
+    const float rstd = 1.0f / sqrtf(ss / (float)gs + eps);
+#pragma unroll
+    for (int it = 0; it < NITER; ++it) {
+        const int j = (it * LANES + lane) * 8;
+        if (j < gs) {
+            float o8[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o8[e] = v[it][e] * rstd;
+            if (w != nullptr) {
+                float wt[8];
+                ld8(w, w_dt, (size_t)g * gs + j, wt);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o8[e] *= wt[e];
+            }
+            if (gate != nullptr && !gate_before) {
+                float gt[8];
+                ld8(gate, gate_dt, gb + j, gt);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o8[e] *= act_f(gt[e], gate_act);
+            }
+            st8(out, out_dt, ob + j, o8);
+        }
+    }
+}
+
 extern "C" int ilm_group_norm_gate(void* out, const void* x, const void* gate, const void* w, int rows, int n, int groups,
                                    int x_stride, int gate_stride, int out_stride, float eps, int gate_act, int gate_before,
                                    int out_dt, int x_dt, int gate_dt, int w_dt, int parts, long pstride, hipStream_t stream) {
     ILM_REQUIRE(parts >= 1, "group_norm_gate: %d parts", parts);
     ILM_REQUIRE(rows > 0 && n > 0 && groups > 0 && n % groups == 0, "group_norm_gate: %d elements do not divide into %d groups", n, groups);
     ILM_REQUIRE((long)rows * groups < (1L << 31) - 4, "group_norm_gate: too many rows");
+    const int gs_ = n / groups;
+    const bool al = gs_ % 8 == 0 && x_stride % 8 == 0 && out_stride % 8 == 0 && (gate == nullptr || gate_stride % 8 == 0) && pstride % 8 == 0
+                    && (((uintptr_t)out | (uintptr_t)x | (uintptr_t)gate | (uintptr_t)w) & 15) == 0;
+    if (al && gs_ <= 8192) {
+#define GN_ARGS out, x, gate, w, rows, n, groups, x_stride, gate_stride, out_stride, eps, gate_act, gate_before, out_dt, x_dt, gate_dt, \
+                w_dt, parts, (size_t)pstride
+        if (gs_ <= 512) group_norm_gate_vec_kernel<64, 1><<<(rows * groups + 3) / 4, 256, 0, stream>>>(GN_ARGS);
+        else if (gs_ <= 2048) group_norm_gate_vec_kernel<256, 1><<<rows * groups, 256, 0, stream>>>(GN_ARGS);
+        else if (gs_ <= 4096) group_norm_gate_vec_kernel<256, 2><<<rows * groups, 256, 0, stream>>>(GN_ARGS);
+        else group_norm_gate_vec_kernel<256, 4><<<rows * groups, 256, 0, stream>>>(GN_ARGS);
+#undef GN_ARGS
+        ILM_LAUNCH_CHECK("group_norm_gate");
+        return 0;
+    }
     if (n / groups > 512) {
         group_norm_gate_kernel<256><<<rows * groups, 256, 0, stream>>>(out, x, gate, w, rows, n, groups, x_stride, gate_stride,
                                                                        out_stride, eps, gate_act, gate_before, out_dt, x_dt, gate_dt, w_dt, parts, (size_t)pstride);
@@ -602,30 +761,6 @@ norm_add_norm_kernel(void* __restrict__ x, float* __restrict__ r, const void* __
     }
     const float rs = 1.0f / sqrtf(block_sum<4>(ss, red) / (float)H + eps);
     for (int j = threadIdx.x; j < H; j += 256) stf(x, x_dt, base + j, r[base + j] * rs * ldf(w, w_dt, j));
-}
-
-// eight consecutive elements as floats / from floats (16-byte accesses for bfloat16, two for float)
-__device__ __forceinline__ void ld8(const void* p, int dt, size_t i, float (&v)[8]) {
-    if (dt == ILM_DTYPE_F32) {
-        const float4 a = *reinterpret_cast<const float4*>((const float*)p + i), b = *reinterpret_cast<const float4*>((const float*)p + i + 4);
-        v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-    } else {
-        uint16_t t[8];
-        *reinterpret_cast<uint4*>(t) = *reinterpret_cast<const uint4*>((const uint16_t*)p + i);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) v[e] = bf16_bits_to_f32(t[e]);
-    }
-}
-__device__ __forceinline__ void st8(void* p, int dt, size_t i, const float (&v)[8]) {
-    if (dt == ILM_DTYPE_F32) {
-        *reinterpret_cast<float4*>((float*)p + i) = make_float4(v[0], v[1], v[2], v[3]);
-        *reinterpret_cast<float4*>((float*)p + i + 4) = make_float4(v[4], v[5], v[6], v[7]);
-    } else {
-        uint16_t t[8];
-#pragma unroll
-        for (int e = 0; e < 8; ++e) t[e] = __builtin_bit_cast(uint16_t, (__bf16)v[e]);
-        *reinterpret_cast<uint4*>((uint16_t*)p + i) = *reinterpret_cast<uint4*>(t);
-    }
 }
 
 // The same for widths that are multiples of 8 up to 8 * 256 * NITER: a thread keeps its pieces of the row in registers
