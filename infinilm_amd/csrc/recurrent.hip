@@ -875,6 +875,7 @@ causal_conv_kernel(float* __restrict__ y, const void* __restrict__ x, const void
 
 // Eight channels a thread (16-byte loads of the inputs, 32-byte stores): channels and the row stride in multiples of 8,
 // bfloat16 inputs, rows 16 bytes aligned.  The taps of a thread's eight channels are 8 * taps consecutive weights.
+template <int TAPS>
 __global__ void __launch_bounds__(256)
 causal_conv_vec_kernel(float* __restrict__ y, const uint16_t* __restrict__ x, const void* __restrict__ w, const void* __restrict__ b,
                        const float* __restrict__ pool, const int* __restrict__ state_in, const int* __restrict__ seg_of_token,
@@ -885,22 +886,22 @@ causal_conv_vec_kernel(float* __restrict__ y, const uint16_t* __restrict__ x, co
     const int r = seg_of_token[t];
     const int j = t - seg_offsets[r];
     const size_t sin = (size_t)state_in[r] * (taps - 1) * C;
-    float s[8];
+    float s[8], wt[TAPS][8];     // wt[m][.]: the weights c * TAPS + 8 m ... of the thread's 8 * TAPS consecutive ones
     if (b != nullptr) ld8(b, w_dt, c, s);
     else {
 #pragma unroll
         for (int e = 0; e < 8; ++e) s[e] = 0.f;
     }
 #pragma unroll
-    for (int i = 0; i < CV_MAX_TAPS; ++i) {
-        if (i < taps) {
-            const int back = taps - 1 - i;
-            float xv[8];
-            if (back <= j) ld8(x, ILM_DTYPE_BF16, (size_t)(t - back) * x_stride + c, xv);
-            else ld8(pool, ILM_DTYPE_F32, sin + (size_t)(taps - 1 - (back - j)) * C + c, xv);
+    for (int m = 0; m < TAPS; ++m) ld8(w, w_dt, (size_t)c * TAPS + 8 * m, wt[m]);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) s[e] = fmaf(ldf(w, w_dt, (size_t)(c + e) * taps + i), xv[e], s[e]);
-        }
+    for (int i = 0; i < TAPS; ++i) {
+        const int back = TAPS - 1 - i;
+        float xv[8];
+        if (back <= j) ld8(x, ILM_DTYPE_BF16, (size_t)(t - back) * x_stride + c, xv);
+        else ld8(pool, ILM_DTYPE_F32, sin + (size_t)(TAPS - 1 - (back - j)) * C + c, xv);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s[e] = fmaf(wt[(e * TAPS + i) / 8][(e * TAPS + i) % 8], xv[e], s[e]);
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e) s[e] = act_f(s[e], act);
@@ -937,13 +938,18 @@ extern "C" int ilm_causal_conv(void* y, const void* x, const void* w, const void
                                int taps, int x_stride, int y_stride, int act, int x_dt, int w_dt, hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && R > 0 && C > 0 && R <= 65535, "causal_conv: bad sizes");
     ILM_REQUIRE(taps >= 1 && taps <= CV_MAX_TAPS, "causal_conv: %d taps, at most %d", taps, CV_MAX_TAPS);
-    const bool vec = x_dt == ILM_DTYPE_BF16 && C % 8 == 0 && x_stride % 8 == 0 && y_stride % 8 == 0
+    // (few rows, decoded tokens: one channel a thread gives more blocks and measured faster: 5.4 against 6.9 us at 64 rows)
+    const bool vec = T_ >= 256 && taps >= 2 && taps <= 4 && ((uintptr_t)w & 15) == 0 && x_dt == ILM_DTYPE_BF16 && C % 8 == 0 && x_stride % 8 == 0 && y_stride % 8 == 0
                      && (((uintptr_t)x | (uintptr_t)y | (uintptr_t)pool | (uintptr_t)b) & 15) == 0;
     for (int t0 = 0; vec && t0 < T_; t0 += 65535) {
         const int rows = T_ - t0 < 65535 ? T_ - t0 : 65535;
-        causal_conv_vec_kernel<<<dim3((C / 8 + 255) / 256, rows), 256, 0, stream>>>(
-            (float*)y, (const uint16_t*)x, w, b, (const float*)pool, (const int*)state_in, (const int*)seg_of_token,
-            (const int*)seg_offsets, C, taps, x_stride, y_stride, act, w_dt, t0);
+#define CV_ARGS (float*)y, (const uint16_t*)x, w, b, (const float*)pool, (const int*)state_in, (const int*)seg_of_token,   \
+                (const int*)seg_offsets, C, taps, x_stride, y_stride, act, w_dt, t0
+        const dim3 vg((C / 8 + 255) / 256, rows);
+        if (taps == 2) causal_conv_vec_kernel<2><<<vg, 256, 0, stream>>>(CV_ARGS);
+        else if (taps == 3) causal_conv_vec_kernel<3><<<vg, 256, 0, stream>>>(CV_ARGS);
+        else causal_conv_vec_kernel<4><<<vg, 256, 0, stream>>>(CV_ARGS);
+#undef CV_ARGS
     }
     for (int t0 = 0; !vec && t0 < T_; t0 += 65535) {
         const int rows = T_ - t0 < 65535 ? T_ - t0 : 65535;
