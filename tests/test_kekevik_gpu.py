@@ -125,6 +125,35 @@ def test_causal_conv_carries_its_last_inputs(taps):
             at += c - a
 
 
+@pytest.mark.parametrize("taps", [2, 3, 4])
+def test_causal_conv_of_long_bfloat16_portions(taps):
+    """Portions of hundreds of tokens in bfloat16 take the form with eight channels a thread: two launches (300 and 280
+    tokens in two segments each, the second from the states the first left) against the convolution over the whole."""
+    from infinilm_amd import kernels
+    C, lens_a, lens_b = 40, [200, 100], [277, 3]
+    g = torch.Generator().manual_seed(10 + taps)
+    w = torch.randn(C, taps, generator=g).to(torch.bfloat16)
+    b = torch.randn(C, generator=g).to(torch.bfloat16)
+    xs = [torch.randn(a + c, C, generator=g).to(torch.bfloat16) for a, c in zip(lens_a, lens_b)]
+    want = []
+    for x in xs:
+        pad = torch.cat([torch.zeros(taps - 1, C), x.float()]).double()
+        want.append(K.silu(torch.stack([(pad[t:t + taps] * w.double().T).sum(0) for t in range(len(x))]) + b.double()))
+    pool = torch.zeros((4, taps - 1, C), device=DEV)
+    rows = torch.tensor([2, 1], dtype=torch.int32, device=DEV)
+    for phase, lens in enumerate([lens_a, lens_b]):
+        cut = [(0, lens_a[r]) if phase == 0 else (lens_a[r], lens_a[r] + lens_b[r]) for r in range(2)]
+        x = torch.cat([xs[r][a:c] for r, (a, c) in enumerate(cut)]).to(DEV)
+        offs = torch.tensor([0, lens[0], sum(lens)], dtype=torch.int32, device=DEV)
+        seg = torch.tensor([r for r, n in enumerate(lens) for _ in range(n)], dtype=torch.int32, device=DEV)
+        sin = torch.zeros(2, dtype=torch.int32, device=DEV) if phase == 0 else rows
+        y = kernels.causal_conv(x, w.to(DEV), b.to(DEV), pool, sin, rows, seg, offs, 2, "silu")
+        at = 0
+        for r, (a, c) in enumerate(cut):
+            _close(y[at:at + c - a].cpu(), want[r][a:c], 1e-5, f"taps {taps} segment {r} phase {phase}")
+            at += c - a
+
+
 def test_group_norm_gate_forms():
     from infinilm_amd import kernels
     g = torch.Generator().manual_seed(2)
