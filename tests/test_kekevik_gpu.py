@@ -362,6 +362,52 @@ def test_recorded_decode_steps_equal_eager_ones(case):
         assert err < case["tol"][r], f"{r}: {err:.3e}"
 
 
+def test_wide_layers_whose_products_come_in_parts(tmp_path):
+    """Layers wide enough for the products that split K over workgroups (their float32 parts go unsummed into the norm
+    that follows a sublayer): a portion of 70 tokens, one of 24, then tokens one by one, in bfloat16."""
+    from infinilm_amd import kernels
+    cfg = {"architecture": "Kekevik", "vocab": 300, "width": 2048, "embedding": {"scale": 4.0}, "norm": {"eps": 1e-6}, "layers": [
+        K._layer("lightning", {"heads": 16, "dim": 128, "vdim": 128, "decay": [1.0 - 2.0 ** -(3 + h // 2) for h in range(16)]}, 8192),
+        K._layer("retention", {"heads": 8, "dim": 64, "vdim": 256, "decay": [0.96875] * 4 + [0.998046875] * 4,
+                               "rot": {"dims": 32, "base": 1e4}}, 8192)]}
+    W = make_dir(str(tmp_path), cfg, 21, "bfloat16")
+    toks = tokens(cfg, 100, 5)
+    want = K.forward(cfg, W, toks)
+    bound = max(TOL["bfloat16"], 2.0 * rel_err(K.forward(cfg, W, toks, round_products=torch.bfloat16), want))
+    drv = Driver(str(tmp_path), "bfloat16", num_pages=4, page_size=64, max_requests=2)
+    kernels.enable_timing(True)
+    drv.step([("a", toks[:70])])
+    drv.step([("a", toks[70:94])])
+    for t in toks[94:]:
+        drv.step([("a", [t])])
+    calls = {k: v["calls"] for k, v in kernels.timing_report().items()}
+    kernels.enable_timing(False)
+    assert calls.get("ilm_gemm_tall", 0) > 0 and calls.get("ilm_gemm_ksplit", 0) > 0, f"the split products did not run: {calls}"
+    err = rel_err(drv.request_logits("a", 100), want)
+    assert err < bound, f"error {err:.3e} (bound {bound:.3e})"
+
+
+def test_norms_of_rows_that_come_in_parts():
+    from infinilm_amd import kernels
+    g = torch.Generator().manual_seed(8)
+    for H in (48, 2048, 4100):
+        parts, r = torch.randn(3, 5, H, generator=g), torch.randn(5, H, generator=g)
+        wb, w = torch.randn(H, generator=g), torch.randn(H, generator=g)
+        y = parts.double().sum(0)
+        res = r.double() + 0.5 * K.rms_unit(y, 1e-5) * wb.double()
+        rd = r.clone().to(DEV)
+        x = kernels.norm_add_norm(rd, parts.to(DEV), wb.to(DEV), 1e-5, 0.5, w.to(DEV), 1e-6, torch.float32)
+        _close(rd.cpu(), res, 1e-5, f"residual, width {H}")
+        _close(x.cpu(), K.rms_unit(res, 1e-6) * w.double(), 1e-5, f"normed rows, width {H}")
+        _close(kernels.group_norm_gate(parts.to(DEV), wb.to(DEV), 1e-5, 1).cpu(), K.rms_unit(y, 1e-5) * wb.double(), 1e-5, f"norm of parts, width {H}")
+        one = parts[0].to(torch.bfloat16)
+        rd = r.clone().to(DEV)
+        x = kernels.norm_add_norm(rd, one.to(DEV), wb.to(torch.bfloat16).to(DEV), 1e-5, 1.0, w.to(torch.bfloat16).to(DEV), 1e-6, torch.bfloat16)
+        res = r.double() + K.rms_unit(one.double(), 1e-5) * wb.to(torch.bfloat16).double()
+        _close(rd.cpu(), res, 1e-5, f"residual from bfloat16 rows, width {H}")
+        _close(x.cpu(), K.rms_unit(res, 1e-6) * w.to(torch.bfloat16).double(), 1e-2, f"bfloat16 normed rows, width {H}")
+
+
 # ---- the entry point and its scheduler ------------------------------------------------------------------------------------
 @pytest.mark.parametrize("name,graph", [("A", False), ("B", False), ("B", True), ("C", True)])
 def test_greedy_generation_through_the_entry_point(name, graph, tmp_path):
