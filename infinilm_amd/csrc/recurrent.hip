@@ -381,7 +381,7 @@ decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__
 // memory once a tile, not once a token.  Thread (kp, column group) owns the SC_NK consecutive state entries
 // kp * SC_NK ... of its VC columns.  LDS: 2 buffers x TB x (2 dkp + columns + 2) floats, dkp = KP * SC_NK.
 template <int MODE, int VC>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3)))   // (three blocks a compute unit: 168 registers)
 decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __restrict__ q, const float* __restrict__ k,
                         int qk_stride, int q_div, const float* __restrict__ v, int v_stride,
                         const float* __restrict__ decay_h, const float* __restrict__ decay_t,
@@ -457,6 +457,7 @@ decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __rest
         if (more) SCT_FETCH(tb + TB)
         const float* b_ = lds + buf * per;
         const int n = min(TB, t1 - tb);
+#pragma unroll 2
         for (int tt = 0; tt < n; ++tt) {
             float qc[SC_NK], kc[SC_NK], vcur[VC];
             const float a = b_[TB * (2 * dkp + cols) + tt], bsc = b_[TB * (2 * dkp + cols + 1) + tt];
