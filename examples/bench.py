@@ -6,7 +6,7 @@ the reference's examples/bench.py (case grid :100-160, one timed generate per ca
         --output-len 64 [--dtype bfloat16] [--enable-graph] [--block-size 64] [--warmup]
     python examples/bench.py --shape 0.5b --batch-size 64 --prompt-len-range 128,2048 --output-len 128 ...
 
-`--shape 8b|0.5b|2b` stands for --model with --skip-load: one of the benchmark shapes of
+`--shape 8b|0.5b|2b|kekevik-1024|kekevik-4096` stands for --model with --skip-load: one of the benchmark shapes of
 examples/shapes.py with random weights.  Prompts are random token ids (no tokenizer is needed) of
 the asked length, or, with `--prompt-len-range LO,HI`, of lengths drawn uniformly from [LO, HI]
 with the case's seed, one length a request (a mixed load: portions of long prompts run beside the
@@ -34,16 +34,18 @@ def int_list(text) -> list:
 
 
 def test_cases(cfg_json: dict, batch_sizes, input_lens, output_lens):
-    """Cases in ascending order of the bytes of cache they fill (bfloat16 keys and values)."""
-    heads = cfg_json["num_attention_heads"]
-    d = cfg_json.get("head_dim") or cfg_json["hidden_size"] // heads
-    nkv = cfg_json.get("num_key_value_heads") or heads
-    layers = cfg_json["num_hidden_layers"]
+    """Cases in ascending order of the bytes of cache they fill (bfloat16 keys and values of every layer that keeps them,
+    whatever the architecture: read off the model's description)."""
+    from infinilm_amd.cache.needs import PagedKV
+    from infinilm_amd.engine.loading import build_model
+    needs = build_model(cfg_json, "bfloat16", "meta").cache_needs
+    flat = [m for n in needs for m in (n if isinstance(n, (tuple, list)) else (n,))]
+    per_token = sum(2 * 2 * m.num_kv_heads * m.head_dim for m in flat if isinstance(m, PagedKV))
     cases = []
     for b in batch_sizes:
         for i in input_lens:
             for o in output_lens:
-                nbytes = 2 * 2 * b * (i + o) * nkv * d * layers
+                nbytes = b * (i + o) * per_token
                 cases.append((nbytes, {"batch_size": b, "input_len": i, "output_len": o,
                                        "kvcache_gb": round(nbytes / 2 ** 30, 3)}))
     return [c for _, c in sorted(cases, key=lambda nc: nc[0])]
@@ -118,7 +120,7 @@ def run_case(llm: LLM, case: dict, seed: int, sp_kwargs: dict) -> dict:
 def main(argv=None) -> int:
     import argparse
     extra = argparse.ArgumentParser(add_help=False)
-    extra.add_argument("--shape", choices=["8b", "0.5b", "2b"], default=None)
+    extra.add_argument("--shape", choices=["8b", "0.5b", "2b", "kekevik-1024", "kekevik-4096"], default=None)
     extra.add_argument("--layers", type=int, default=0, help="with --shape: run this many layers instead of the shape's")
     extra.add_argument("--prompt-len-range", type=str, default=None, help="LO,HI: a length of its own for every request")
     ex, rest = extra.parse_known_args(sys.argv[1:] if argv is None else argv)

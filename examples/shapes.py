@@ -13,7 +13,11 @@ def _factors(n: int, seed: int):
 
 
 def shape_config(name: str, layers: int = 0) -> dict:
-    """`name`: "8b", "0.5b" or "2b"; `layers` > 0 overrides the number of layers."""
+    """`name`: "8b", "0.5b", "2b" (MiniCPM4 family) or "kekevik-<width>" (the Kekevik design at that width, 8 layers unless
+    told otherwise); `layers` > 0 overrides the number of layers."""
+    if name.startswith("kekevik-"):
+        width = int(name.split("-")[1])
+        return kekevik_shape(width, width // 128, 128, 2, layers or 8, 32768, 6 * width)
     base = {"architectures": ["MiniCPMForCausalLM"], "model_type": "minicpm", "torch_dtype": "bfloat16", "rope_theta": 10000.0,
             "scale_emb": 12, "scale_depth": 1.4, "dim_model_base": 256}
     if name == "8b":

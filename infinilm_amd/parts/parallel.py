@@ -1,4 +1,5 @@
-"""Mixers side by side: every branch reads the same input, the result is the weighted sum of their outputs.
+"""Mixers side by side: every branch reads the same input, the result is the weighted sum of their outputs (float32:
+it goes to a norm or into the residual sum, not into a product).
 
 `branches` are mixers of any registered kind, `scales` their weights, `names` the sub-names of their tensors.  What
 the branches need of the cache is handed on as one tuple (a branch that itself needs a tuple takes as many members),
@@ -7,6 +8,8 @@ and the views come back in the same order.
 from __future__ import annotations
 
 from typing import Dict, List, Sequence
+
+import torch
 
 from .. import kernels
 from ..config.spec import PartSpec
@@ -64,9 +67,9 @@ class ParallelMixers(Mixer):
             if total is None:
                 total, first = y, s
             elif first is not None:
-                total, first = kernels.weighted_sum(total, y, first, s, out_dtype=self.dtype), None
+                total, first = kernels.weighted_sum(total, y, first, s, out_dtype=torch.float32), None
             else:
-                total = kernels.weighted_sum(total, y, 1.0, s, out_dtype=self.dtype)
+                total = kernels.weighted_sum(total, y, 1.0, s, out_dtype=torch.float32)
         if first is not None:    # a single branch
-            total = kernels.weighted_sum(total, total, first, 0.0, out_dtype=self.dtype)
+            total = kernels.weighted_sum(total, total, first, 0.0, out_dtype=torch.float32)
         return total
