@@ -1066,26 +1066,23 @@ weighted_sum_kernel(void* __restrict__ out, const void* __restrict__ x, const vo
 }
 
 __global__ void __launch_bounds__(256)
-weighted_sum_vec_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ x, const uint16_t* __restrict__ y, long n,
-                        float a, float b) {
+weighted_sum_vec_kernel(void* __restrict__ out, const void* __restrict__ x, const void* __restrict__ y, long n, float a, float b,
+                        int out_dt, int x_dt, int y_dt) {
     const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 8;
     if (i >= n) return;
-    uint16_t p[8], q[8], r[8];
-    *reinterpret_cast<uint4*>(p) = *reinterpret_cast<const uint4*>(x + i);
-    *reinterpret_cast<uint4*>(q) = *reinterpret_cast<const uint4*>(y + i);
+    float p[8], q[8], r[8];
+    ld8(x, x_dt, i, p);
+    ld8(y, y_dt, i, q);
 #pragma unroll
-    for (int e = 0; e < 8; ++e)
-        r[e] = __builtin_bit_cast(uint16_t, (__bf16)fmaf(a, bf16_bits_to_f32(p[e]), b * bf16_bits_to_f32(q[e])));
-    *reinterpret_cast<uint4*>(out + i) = *reinterpret_cast<uint4*>(r);
+    for (int e = 0; e < 8; ++e) r[e] = fmaf(a, p[e], b * q[e]);
+    st8(out, out_dt, i, r);
 }
 
 extern "C" int ilm_weighted_sum(void* out, const void* x, const void* y, long n, float a, float b, int out_dt, int x_dt,
                                 int y_dt, hipStream_t stream) {
     ILM_REQUIRE(n > 0 && (n + 255) / 256 < (1L << 31), "weighted_sum: bad size");
-    if (out_dt == ILM_DTYPE_BF16 && x_dt == ILM_DTYPE_BF16 && y_dt == ILM_DTYPE_BF16 && n % 8 == 0 && ((uintptr_t)out & 15) == 0
-        && ((uintptr_t)x & 15) == 0 && ((uintptr_t)y & 15) == 0) {
-        weighted_sum_vec_kernel<<<(unsigned)((n / 8 + 255) / 256), 256, 0, stream>>>((uint16_t*)out, (const uint16_t*)x,
-                                                                                     (const uint16_t*)y, n, a, b);
+    if (n % 8 == 0 && (((uintptr_t)out | (uintptr_t)x | (uintptr_t)y) & 15) == 0) {
+        weighted_sum_vec_kernel<<<(unsigned)((n / 8 + 255) / 256), 256, 0, stream>>>(out, x, y, n, a, b, out_dt, x_dt, y_dt);
         ILM_LAUNCH_CHECK("weighted_sum");
         return 0;
     }
