@@ -27,7 +27,7 @@ ARCH = "gfx950"
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-result", "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument",
+    "-Wno-unused-result", "-Wno-unknown-warning-option", "-Wno-unused-command-line-argument", "-Wno-pass-failed",
 ]
 
 

@@ -250,7 +250,6 @@ __device__ __forceinline__ float sc_fold4(const float (&acc)[4], int kp, int KP)
 }
 
 #define SC_NK 8
-#define SC_WHOLE 0
 #define SC_LOCAL 1
 #define SC_FROM 2
 
@@ -266,55 +265,40 @@ __device__ __forceinline__ int sc_find(const int* __restrict__ seg_offsets, int 
     return (p >= 0 && p * piece < len) ? lo : -1;
 }
 
-template <int MODE, int VC>   // VC: value columns a thread (the q and k a thread loads serve all of them)
+template <int VC>   // VC: value columns a thread (the q and k a thread loads serve all of them)
 __global__ void __launch_bounds__(256)
 decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__ q, const float* __restrict__ k,
                   int qk_stride, int q_div, const float* __restrict__ v, int v_stride,
                   const float* __restrict__ decay_h, const float* __restrict__ decay_t,
                   const float* __restrict__ kscale_t, const float* __restrict__ skip_h, float* __restrict__ pool,
                   const int* __restrict__ state_in, const int* __restrict__ state_out,
-                  const int* __restrict__ seg_offsets, int heads, int dk, int dv, int KP, int R, int piece,
-                  float* __restrict__ ws_state, float* __restrict__ ws_decay) {
-    const int h = blockIdx.y;
-    int r, t0, t1, slot = 0;
-    if (MODE == SC_WHOLE) {
-        r = blockIdx.z;
-        t0 = seg_offsets[r];
-        t1 = seg_offsets[r + 1];
-        if (t0 >= t1) return;
-    } else {
-        int p;
-        slot = blockIdx.z;
-        r = sc_find(seg_offsets, R, piece, slot, p);
-        if (r < 0) return;
-        t0 = seg_offsets[r] + p * piece;
-        t1 = min(t0 + piece, seg_offsets[r + 1]);
-    }
+                  const int* __restrict__ seg_offsets, int heads, int dk, int dv, int KP) {
+    const int h = blockIdx.y, r = blockIdx.z;
+    const int t0 = seg_offsets[r], t1 = seg_offsets[r + 1];
+    if (t0 >= t1) return;
     const int VT = 256 / KP;                                 // column groups a block
     const int kp = threadIdx.x % KP, vc0 = (blockIdx.x * VT + threadIdx.x / KP) * VC;
     const size_t hs = (size_t)dk * dv;                       // floats of a head's state
-    const float* src = MODE == SC_WHOLE ? pool + ((size_t)state_in[r] * heads + h) * hs
-                                        : ws_state + ((size_t)slot * heads + h) * hs;
+    const float* src = pool + ((size_t)state_in[r] * heads + h) * hs;
     float S[VC][SC_NK];
 #pragma unroll
     for (int c = 0; c < VC; ++c)
 #pragma unroll
         for (int i = 0; i < SC_NK; ++i) {
             const int ki = i * KP + kp;
-            S[c][i] = (MODE != SC_LOCAL && vc0 + c < dv && ki < dk) ? src[(size_t)(vc0 + c) * dk + ki] : 0.f;
+            S[c][i] = (vc0 + c < dv && ki < dk) ? src[(size_t)(vc0 + c) * dk + ki] : 0.f;
         }
     const int qoff = (h / q_div) * dk;
     const float a_h = decay_h != nullptr ? decay_h[h] : 1.0f;
     const float skip = skip_h != nullptr ? skip_h[h] : 0.f;
     float qn[SC_NK], kn[SC_NK], vn[VC], an, bn;
-    float aprod = 1.0f;
 #define SC_LOAD(T_)                                                                              \
     {                                                                                            \
         const float* qr = q + (size_t)(T_) * qk_stride + qoff;                                   \
         const float* kr = k + (size_t)(T_) * qk_stride + qoff;                                   \
         _Pragma("unroll") for (int i = 0; i < SC_NK; ++i) {                                      \
             const int ki = i * KP + kp;                                                          \
-            if (MODE != SC_LOCAL) qn[i] = ki < dk ? qr[ki] : 0.f;                                \
+            qn[i] = ki < dk ? qr[ki] : 0.f;                                                      \
             kn[i] = ki < dk ? kr[ki] : 0.f;                                                      \
         }                                                                                        \
         _Pragma("unroll") for (int c = 0; c < VC; ++c)                                           \
@@ -328,12 +312,12 @@ decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__
         const float a = an, b = bn;
 #pragma unroll
         for (int i = 0; i < SC_NK; ++i) {
-            if (MODE != SC_LOCAL) qc[i] = qn[i];
+            qc[i] = qn[i];
             kc[i] = kn[i] * b;
         }
 #pragma unroll
         for (int c = 0; c < VC; ++c) vcur[c] = vn[c];
-        if (t + 1 < t1) SC_LOAD(t + 1)
+        if (t + 1 < t1) SC_LOAD(t + 1)      // the next token's operands are on their way while this one is computed
         float acc[VC];
 #pragma unroll
         for (int c = 0; c < VC; ++c) {
@@ -341,30 +325,25 @@ decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__
 #pragma unroll
             for (int i = 0; i < SC_NK; ++i) {
                 S[c][i] = fmaf(a, S[c][i], kc[i] * vcur[c]);
-                if (MODE != SC_LOCAL) acc[c] = fmaf(S[c][i], qc[i], acc[c]);
+                acc[c] = fmaf(S[c][i], qc[i], acc[c]);
             }
         }
-        if (MODE == SC_LOCAL) {
-            aprod *= a;
+        if (VC == 4 && KP >= 4) {
+            const float (&a4)[4] = reinterpret_cast<const float (&)[4]>(acc);
+            const float tot = sc_fold4(a4, kp, KP);
+            const int c = 2 * (kp & 1) + ((kp >> 1) & 1);
+            const float vsel = c == 0 ? vcur[0] : c == 1 ? vcur[VC > 1 ? 1 : 0] : c == 2 ? vcur[VC > 2 ? 2 : 0] : vcur[VC > 3 ? 3 : 0];
+            if (kp < 4 && vc0 + c < dv) o[(size_t)t * o_stride + (size_t)h * dv + vc0 + c] = fmaf(skip, vsel, tot);
         } else {
-            if (VC == 4 && KP >= 4) {
-                const float (&a4)[4] = reinterpret_cast<const float (&)[4]>(acc);
-                const float tot = sc_fold4(a4, kp, KP);
-                const int c = 2 * (kp & 1) + ((kp >> 1) & 1);
-                const float vsel = c == 0 ? vcur[0] : c == 1 ? vcur[VC > 1 ? 1 : 0] : c == 2 ? vcur[VC > 2 ? 2 : 0] : vcur[VC > 3 ? 3 : 0];
-                if (kp < 4 && vc0 + c < dv) o[(size_t)t * o_stride + (size_t)h * dv + vc0 + c] = fmaf(skip, vsel, tot);
-            } else {
 #pragma unroll
-                for (int c = 0; c < VC; ++c) {
-                    for (int off = 1; off < KP; off <<= 1) acc[c] += __shfl_xor(acc[c], off, 64);
-                    if (kp == 0 && vc0 + c < dv) o[(size_t)t * o_stride + (size_t)h * dv + vc0 + c] = fmaf(skip, vcur[c], acc[c]);
-                }
+            for (int c = 0; c < VC; ++c) {
+                for (int off = 1; off < KP; off <<= 1) acc[c] += __shfl_xor(acc[c], off, 64);
+                if (kp == 0 && vc0 + c < dv) o[(size_t)t * o_stride + (size_t)h * dv + vc0 + c] = fmaf(skip, vcur[c], acc[c]);
             }
         }
     }
 #undef SC_LOAD
-    if (MODE == SC_FROM) return;
-    float* dst = MODE == SC_WHOLE ? pool + ((size_t)state_out[r] * heads + h) * hs : ws_state + ((size_t)slot * heads + h) * hs;
+    float* dst = pool + ((size_t)state_out[r] * heads + h) * hs;
 #pragma unroll
     for (int c = 0; c < VC; ++c)
 #pragma unroll
@@ -372,10 +351,9 @@ decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__
             const int ki = i * KP + kp;
             if (vc0 + c < dv && ki < dk) dst[(size_t)(vc0 + c) * dk + ki] = S[c][i];
         }
-    if (MODE == SC_LOCAL && blockIdx.x == 0 && threadIdx.x == 0) ws_decay[(size_t)slot * heads + h] = aprod;
 }
 
-// The pieces' form of the kernel above (SC_LOCAL, SC_FROM): a token's q, k, v, decay and scale reach the threads through
+// The pieces' form (SC_LOCAL: local states, SC_FROM: outputs from given start states): a token's q, k, v, decay and scale reach the threads through
 // LDS in tiles of TB tokens that the block loads together, the next tile on its way from memory while this one is
 // computed (one barrier a tile), instead of every thread loading its own entries token by token: a wave then waits for
 // memory once a tile, not once a token.  Thread (kp, column group) owns the SC_NK consecutive state entries
@@ -557,15 +535,14 @@ extern "C" int ilm_decay_scan(void* o, int o_stride, const void* q, const void* 
     const int VT = 256 / KP;
 #define SC_ARGS (float*)o, o_stride, (const float*)q, (const float*)k, qk_stride, q_div, (const float*)v, v_stride,              \
                 (const float*)decay_h, (const float*)decay_t, (const float*)kscale_t, (const float*)skip_h, (float*)pool,        \
-                (const int*)state_in, (const int*)state_out, (const int*)seg_offsets, heads, dk, dv, KP, R, piece,              \
-                (float*)ws_state, (float*)ws_decay
+                (const int*)state_in, (const int*)state_out, (const int*)seg_offsets, heads, dk, dv, KP
     // four columns a thread where that still leaves two blocks a compute unit (long prompts in pieces, large batches):
     // a thread's loads of q and k then serve four columns; one column a thread where blocks are few (small batches)
     const int cus = ilm_num_cus();
     if (piece == 0) {
         const int g4 = (dv + 4 * VT - 1) / (4 * VT);
-        if ((long)g4 * heads * R >= 2L * cus && dv >= 4) decay_scan_kernel<SC_WHOLE, 4><<<dim3(g4, heads, R), 256, 0, stream>>>(SC_ARGS);
-        else decay_scan_kernel<SC_WHOLE, 1><<<dim3((dv + VT - 1) / VT, heads, R), 256, 0, stream>>>(SC_ARGS);
+        if ((long)g4 * heads * R >= 2L * cus && dv >= 4) decay_scan_kernel<4><<<dim3(g4, heads, R), 256, 0, stream>>>(SC_ARGS);
+        else decay_scan_kernel<1><<<dim3((dv + VT - 1) / VT, heads, R), 256, 0, stream>>>(SC_ARGS);
         ILM_LAUNCH_CHECK("decay_scan");
         return 0;
     }

@@ -1021,7 +1021,8 @@ SCAN_PIECE_FROM = int(os.environ.get("INFINILM_AMD_SCAN_PIECE_FROM", "129"))   #
 CONV_MAX_TAPS = 8           # most taps of the short convolution (ilm_causal_conv_max_taps())
 
 
-def _act(kind: str) -> int:
+def activation_code(kind: str) -> int:
+    """The kernels' number of an activation's name; raises for a name they do not know (parts call it when they are built)."""
     try:
         return ACTIVATIONS[kind]
     except KeyError:
@@ -1039,7 +1040,7 @@ def activation(x: torch.Tensor, kind: str, out_dtype: Optional[torch.dtype] = No
     _rows(x, "x")
     T, n = x.shape
     out = torch.empty((T, n), dtype=out_dtype or x.dtype, device=x.device)
-    _run("ilm_unary", out.data_ptr(), x.data_ptr(), T, n, out.stride(0), x.stride(0), _act(kind), _dt(out), _dt(x), _stream())
+    _run("ilm_unary", out.data_ptr(), x.data_ptr(), T, n, out.stride(0), x.stride(0), activation_code(kind), _dt(out), _dt(x), _stream())
     return out
 
 
@@ -1062,7 +1063,7 @@ def linear_attention_inputs(qkv: torch.Tensor, positions: Optional[torch.Tensor]
             raise KernelError(f"frequencies must be float32 [{rotary_dims // 2}] and positions one a token")
     out = torch.empty((T, n), dtype=F32, device=qkv.device)
     _run("ilm_lin_prep", out.data_ptr(), qkv.data_ptr(), _ptr(positions), _ptr(freq), T, heads, dk, dv, int(rotary_dims),
-         qkv.stride(0), _act(act), float(k_scale), _dt(qkv), _stream())
+         qkv.stride(0), activation_code(act), float(k_scale), _dt(qkv), _stream())
     return out
 
 
@@ -1139,7 +1140,7 @@ def group_norm_gate(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
             raise KernelError(f"gate {tuple(gate.shape)} does not match {tuple(x.shape)}")
     out = torch.empty((T, n), dtype=out_dtype or x.dtype, device=x.device)
     _run("ilm_group_norm_gate", out.data_ptr(), x.data_ptr(), _ptr(gate), _ptr(weight), T, n, int(groups), x.stride(0),
-         gate.stride(0) if gate is not None else 0, out.stride(0), float(eps), _act(gate_act), int(bool(gate_before)),
+         gate.stride(0) if gate is not None else 0, out.stride(0), float(eps), activation_code(gate_act), int(bool(gate_before)),
          _dt(out), _dt(x), _dt(gate) if gate is not None else 0, _dt(weight) if weight is not None else 0, parts, pstride,
          _stream())
     return out
@@ -1171,7 +1172,7 @@ def causal_conv(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tens
     y = torch.empty((T, C), dtype=F32, device=x.device)
     _run("ilm_causal_conv", y.data_ptr(), x.data_ptr(), weight.data_ptr(), _ptr(bias), pool.data_ptr(), state_in.data_ptr(),
          state_out.data_ptr(), seg_of_token.data_ptr(), seg_offsets.data_ptr(), T, int(segments), C, taps, x.stride(0),
-         y.stride(0), _act(act), _dt(x), _dt(weight), _stream())
+         y.stride(0), activation_code(act), _dt(x), _dt(weight), _stream())
     return y
 
 

@@ -43,7 +43,7 @@ class DecayLinearAttention(Mixer):
         self.gate_act = gate_act
         self.whole_output = bool(whole_output)    # never float32 parts still to be summed (see GQAttention)
         self.dtype = ctx.dtype
-        kernels._act(activation), kernels._act(gate_act)
+        kernels.activation_code(activation), kernels.activation_code(gate_act)
         qn, kn, vn, gn, on, self.norm_name = names
         self.proj = FusedLinear(hidden_size, [self.H * self.dk, self.H * self.dk, self.H * self.dv, self.H * self.dv],
                                 [qn, kn, vn, gn], False, ctx, suffix=suffix)

@@ -57,7 +57,7 @@ class ActivationMLP(FeedForward):
 
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str, bias: bool, ctx: BuildContext,
                  names=("up_proj", "down_proj"), suffix: str = "weight", whole_output: bool = False):
-        kernels._act(activation)
+        kernels.activation_code(activation)
         self.activation = activation
         self.whole_output = bool(whole_output)
         self.up = Linear(hidden_size, intermediate_size, names[0], bias, ctx, suffix=suffix)
