@@ -20,15 +20,18 @@ class Architecture:
     name: str
     config_from_dict: Callable[[Dict[str, Any]], Any]
     build_spec: Callable[[Any], ModelSpec]
+    # optional: (raw config, {tensor name: shape}) -> raw config completed with the sizes that only a checkpoint's
+    # tensors give; called when the configuration comes from a model folder
+    sizes_from_checkpoint: Any = None
 
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
 
 
-def register_architecture(names: Iterable[str], config_from_dict, build_spec) -> None:
+def register_architecture(names: Iterable[str], config_from_dict, build_spec, sizes_from_checkpoint=None) -> None:
     """`names`: every `architectures` entry and `model_type` value that selects this model."""
     names = list(names)
-    arch = Architecture(names[0], config_from_dict, build_spec)
+    arch = Architecture(names[0], config_from_dict, build_spec, sizes_from_checkpoint)
     for n in names:
         _ARCHITECTURES[n] = arch
 
@@ -78,4 +81,7 @@ def load_model_config(model_dir_or_dict):
 
     raw = model_dir_or_dict if isinstance(model_dir_or_dict, dict) else read_config_json(model_dir_or_dict)
     arch = resolve_architecture(raw)
+    if arch.sizes_from_checkpoint is not None and not isinstance(model_dir_or_dict, dict):
+        from ..weights.loader import checkpoint_shapes
+        raw = arch.sizes_from_checkpoint(raw, checkpoint_shapes(model_dir_or_dict))
     return arch, arch.config_from_dict(raw)

@@ -28,6 +28,15 @@ class LayerSpec:
 
 
 @dataclass(frozen=True)
+class RunStart:
+    """What is added to the residual stream right before a run (a pass over a stretch of layers that opens with it):
+    `embedding` times the embedding's output as it was before the first layer (0: nothing), and row `vector_row` of the
+    model's tensor `ModelSpec.run_vectors` (None: no row)."""
+    embedding: float = 0.0
+    vector_row: Optional[int] = None
+
+
+@dataclass(frozen=True)
 class LayerRun:
     """One entry of the execution order: run `layer` with cache entry `cache`.
 
@@ -36,6 +45,7 @@ class LayerRun:
     layer: int
     cache: Optional[int]
     writes_cache: bool = True
+    start: Optional[RunStart] = None
 
 
 @dataclass
@@ -71,6 +81,8 @@ class ModelSpec:
     # axes of the positions a step carries for every token (1: the place in the sequence alone; a position encoding
     # over several axes, rows and columns of a picture beside the place in the text, reads `batch.position_axes`)
     position_axes: int = 1
+    # (name, rows): a tensor [rows, hidden] of vectors that runs add to the residual stream (`RunStart.vector_row`)
+    run_vectors: Optional[tuple] = None
 
     def num_cache_entries(self) -> int:
         ids = [r.cache for r in self.order if r.cache is not None]
@@ -86,6 +98,11 @@ class ModelSpec:
                 if run.cache in writers:
                     raise ValueError(f"cache entry {run.cache} is written by order[{writers[run.cache]}] and order[{i}]")
                 writers[run.cache] = i
+        for i, run in enumerate(self.order):
+            row = run.start.vector_row if run.start is not None else None
+            if row is not None and (self.run_vectors is None or not 0 <= row < self.run_vectors[1]):
+                raise ValueError(f"order[{i}] adds row {row} of the run vectors, of which there are "
+                                 f"{self.run_vectors[1] if self.run_vectors else 0}")
         for i, run in enumerate(self.order):
             if run.cache is not None and not run.writes_cache:
                 if run.cache not in writers or writers[run.cache] > i:

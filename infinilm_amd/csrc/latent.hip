@@ -1,0 +1,153 @@
+// Attention over a small latent row a token, in its absorbed form: the cache holds, for every token, the normed
+// latent c [rank] and one rotated key part [dr] shared by the heads; a query head's unrotated part is carried into
+// the latent space (q_h^T W_uk,h, a product per head), so that the scores are plain dot products of rows of
+// rank + dr entries against one cached key row, and the values are the latent rows themselves, carried out of the
+// latent space after the attention (W_uv,h times the head's result).  The attention itself is the paged kernels'
+// with one key/value head of d >= rank + dr entries.
+//
+//   ilm_latent_prep   from the fused projection rows [q: H (dn + dr) | down: rank + dr]: c = RMS norm of the first
+//       rank entries of `down` times a weight; the last dr entries and every head's last dr query entries turned
+//       in pairs (2i, 2i + 1) by pos * freq[i]; key row [c | turned part | zeros] and value column [c | zeros] into
+//       the cache; the turned query parts (and zeros behind them) into the attention's query rows [T, H, d].
+//   ilm_head_gemm     out[t, h, n] = sum_k x[t, h, k] W[h, k, n] with strides for every axis (a product per head),
+//       float sums in ascending k whatever the number of rows.
+#include "common.h"
+
+template <typename T, typename TW>
+__global__ void __launch_bounds__(256)
+latent_prep_kernel(const T* __restrict__ rows, T* __restrict__ qx, const int* __restrict__ pos, const float* __restrict__ freq,
+                   const TW* __restrict__ w, T* __restrict__ kc, T* __restrict__ vc, const int* __restrict__ slots,
+                   int H, int dn, int dr, int rank, int d, float eps, int page, int stride) {
+    extern __shared__ float c[];
+    __shared__ float red[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const T* row = rows + (size_t)t * stride;
+    const T* down = row + (size_t)H * (dn + dr);
+    float ss = 0.f;
+    for (int e = tid; e < rank; e += 256) {
+        const float v = to_f32(down[e]);
+        c[e] = v;
+        ss = fmaf(v, v, ss);
+    }
+    const float rstd = 1.0f / sqrtf(block_sum<4>(ss, red) / (float)rank + eps);
+    const float p = (float)pos[t];
+    const int slot = slots != nullptr ? slots[t] : -1;
+    if (slot >= 0) {
+        const int pg = slot / page, off = slot % page;
+        T* kdst = kc + ((size_t)pg * page + off) * d;
+        T* vdst = vc + (size_t)pg * d * page + off;
+        for (int e = tid; e < d; e += 256) {
+            float kv = 0.f, vv = 0.f;
+            if (e < rank) {
+                kv = vv = c[e] * rstd * to_f32(w[e]);
+            } else if (e < rank + dr) {
+                const int i = (e - rank) >> 1;
+                float sn, cs;
+                sincosf(p * freq[i], &sn, &cs);
+                const float u = to_f32(down[rank + 2 * i]), v = to_f32(down[rank + 2 * i + 1]);
+                kv = ((e - rank) & 1) ? v * cs + u * sn : u * cs - v * sn;
+            }
+            kdst[e] = from_f32<T>(kv);
+            vdst[(size_t)e * page] = from_f32<T>(vv);
+        }
+    }
+    // the queries' turned parts and the zeros behind them
+    const int tail = d - rank;
+    for (int idx = tid; idx < H * tail; idx += 256) {
+        const int h = idx / tail, e = idx % tail;
+        float y = 0.f;
+        if (e < dr) {
+            const int i = e >> 1;
+            float sn, cs;
+            sincosf(p * freq[i], &sn, &cs);
+            const T* qr = row + (size_t)h * (dn + dr) + dn;
+            const float u = to_f32(qr[2 * i]), v = to_f32(qr[2 * i + 1]);
+            y = (e & 1) ? v * cs + u * sn : u * cs - v * sn;
+        }
+        qx[((size_t)t * H + h) * d + rank + e] = from_f32<T>(y);
+    }
+}
+
+extern "C" int ilm_latent_prep(const void* rows, void* qx, const void* pos, const void* freq, const void* w, void* kc, void* vc,
+                               const void* slots, int T_, int H, int dn, int dr, int rank, int d, float eps, int page,
+                               int stride, int dtype, int w_dt, hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && H > 0 && dn > 0 && dr >= 0 && rank > 0 && page > 0, "latent_prep: bad sizes");
+    ILM_REQUIRE(dr % 2 == 0 && d >= rank + dr && rank <= 8192, "latent_prep: %d + %d entries in rows of %d", rank, dr, d);
+    ILM_REQUIRE(stride >= H * (dn + dr) + rank + dr, "latent_prep: rows of %d do not hold the projections", stride);
+    ILM_REQUIRE(dr == 0 || freq != nullptr, "latent_prep: a rotation needs frequencies");
+    const size_t shm = (size_t)rank * sizeof(float);
+#define LP_LAUNCH(T__, TW__)                                                                                          \
+    latent_prep_kernel<T__, TW__><<<T_, 256, shm, stream>>>((const T__*)rows, (T__*)qx, (const int*)pos, (const float*)freq, \
+                                                            (const TW__*)w, (T__*)kc, (T__*)vc, (const int*)slots, H, dn, dr, \
+                                                            rank, d, eps, page, stride)
+    if (dtype == ILM_DTYPE_F32 && w_dt == ILM_DTYPE_F32) LP_LAUNCH(float, float);
+    else if (dtype == ILM_DTYPE_BF16 && w_dt == ILM_DTYPE_BF16) LP_LAUNCH(bf16, bf16);
+    else if (dtype == ILM_DTYPE_BF16 && w_dt == ILM_DTYPE_F32) LP_LAUNCH(bf16, float);
+    else ILM_REQUIRE(false, "latent_prep: dtypes %d / %d", dtype, w_dt);
+#undef LP_LAUNCH
+    ILM_LAUNCH_CHECK("latent_prep");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// A product per head.  A block: 16 rows x 64 outputs of one head; x and W pass through LDS in steps of 64 k.
+// Thread (n, row group) holds 4 rows of one output column.  W's fast axis may be k or n; the tile is loaded along it.
+// ------------------------------------------------------------------------------------------
+#define HG_ROWS 16
+#define HG_COLS 64
+#define HG_K 64
+
+template <typename T, typename TO>
+__global__ void __launch_bounds__(256)
+head_gemm_kernel(TO* __restrict__ out, const T* __restrict__ x, const T* __restrict__ w, int M, int N, int K, long x_t, long x_h,
+                 long w_h, long w_k, long w_n, long o_t, long o_h) {
+    __shared__ float xs[HG_ROWS][HG_K + 1];
+    __shared__ float ws[HG_K][HG_COLS + 1];
+    const int h = blockIdx.z, n0 = blockIdx.x * HG_COLS, m0 = blockIdx.y * HG_ROWS, tid = threadIdx.x;
+    const int nl = tid & 63, rg = tid >> 6;
+    const T* xh = x + (size_t)h * x_h;
+    const T* wh = w + (size_t)h * w_h;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < K; k0 += HG_K) {
+        for (int i = tid; i < HG_ROWS * HG_K; i += 256) {
+            const int r = i / HG_K, kk = i % HG_K;
+            xs[r][kk] = (m0 + r < M && k0 + kk < K) ? to_f32(xh[(size_t)(m0 + r) * x_t + k0 + kk]) : 0.f;
+        }
+        for (int i = tid; i < HG_K * HG_COLS; i += 256) {
+            const int kk = w_n == 1 ? i / HG_COLS : i % HG_K, nn = w_n == 1 ? i % HG_COLS : i / HG_K;
+            ws[kk][nn] = (k0 + kk < K && n0 + nn < N) ? to_f32(wh[(size_t)(k0 + kk) * w_k + (size_t)(n0 + nn) * w_n]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int kk = 0; kk < HG_K; ++kk) {
+            const float wv = ws[kk][nl];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[r] = fmaf(xs[rg * 4 + r][kk], wv, acc[r]);
+        }
+        __syncthreads();
+    }
+    if (n0 + nl < N)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int m = m0 + rg * 4 + r;
+            if (m < M) out[(size_t)m * o_t + (size_t)h * o_h + n0 + nl] = from_f32<TO>(acc[r]);
+        }
+}
+
+extern "C" int ilm_head_gemm(void* out, const void* x, const void* w, int M, int N, int K, int H, long x_t, long x_h, long w_h,
+                             long w_k, long w_n, long o_t, long o_h, int dtype, int out_dt, hipStream_t stream) {
+    ILM_REQUIRE(M > 0 && N > 0 && K > 0 && H > 0 && H <= 65535, "head_gemm: bad sizes");
+    ILM_REQUIRE((M + HG_ROWS - 1) / HG_ROWS <= 65535, "head_gemm: too many rows");
+    ILM_REQUIRE(w_k == 1 || w_n == 1, "head_gemm: one axis of W must be dense");
+    dim3 grid((N + HG_COLS - 1) / HG_COLS, (M + HG_ROWS - 1) / HG_ROWS, H);
+#define HG_LAUNCH(T__, TO__)                                                                                              \
+    head_gemm_kernel<T__, TO__><<<grid, 256, 0, stream>>>((TO__*)out, (const T__*)x, (const T__*)w, M, N, K, x_t, x_h, w_h, \
+                                                          w_k, w_n, o_t, o_h)
+    if (dtype == ILM_DTYPE_F32 && out_dt == ILM_DTYPE_F32) HG_LAUNCH(float, float);
+    else if (dtype == ILM_DTYPE_BF16 && out_dt == ILM_DTYPE_BF16) HG_LAUNCH(bf16, bf16);
+    else if (dtype == ILM_DTYPE_BF16 && out_dt == ILM_DTYPE_F32) HG_LAUNCH(bf16, float);
+    else ILM_REQUIRE(false, "head_gemm: dtypes %d / %d", dtype, out_dt);
+#undef HG_LAUNCH
+    ILM_LAUNCH_CHECK("head_gemm");
+    return 0;
+}

@@ -52,7 +52,13 @@ _SIGNATURES = {
     "ilm_sample": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
     "ilm_unary": [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "ilm_lin_prep": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
-    "ilm_decay_scan": [_P, _I, _P, _P, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P],
+    "ilm_decay_scan": [_P, _I, _P, _P, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P],
+    "ilm_sigmoid_root": [_P, _P, _I, _I, _I, _I, _F, _I, _P],
+    "ilm_add_layernorm": [_P, _P, _P, _P, _I, _I, _F, _I, _I, _I] + [_P, _I, _I, _L, _L, _F] * 4 + [_P],
+    "ilm_qkv_norm_rope_kvwrite": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
+    "ilm_attn_headmix": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "ilm_latent_prep": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
+    "ilm_head_gemm": [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _I, _I, _P],
     "ilm_group_norm_gate": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _I, _I, _L, _P],
     "ilm_causal_conv": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P],
     "ilm_ssm_steps": [_P, _P, _P, _P, _P, _I, _I, _I, _I, _P],

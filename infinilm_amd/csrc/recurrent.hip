@@ -109,6 +109,38 @@ extern "C" int ilm_unary(void* out, const void* in, int T_, int n, int out_strid
 }
 
 // ------------------------------------------------------------------------------------------
+// Decays of a gated recurrence from their raw rows: out[t, j] = sigmoid(z[t, j])^inv_tau = exp(inv_tau * log sigmoid(z)),
+// the logarithm in its stable form (-log1p(exp(-z)) for z >= 0, z - log1p(exp(z)) below); float results.
+// ------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256)
+sigmoid_root_kernel(float* __restrict__ out, const T* __restrict__ z, int n, int out_stride, int in_stride, float inv_tau) {
+    const int t = blockIdx.y, j = blockIdx.x * 256 + threadIdx.x;
+    if (j >= n) return;
+    const float x = to_f32(z[(size_t)t * in_stride + j]);
+    const float ls = x >= 0.f ? -log1pf(expf(-x)) : x - log1pf(expf(x));
+    out[(size_t)t * out_stride + j] = expf(inv_tau * ls);
+}
+
+extern "C" int ilm_sigmoid_root(void* out, const void* z, int T_, int n, int out_stride, int in_stride, float inv_tau, int z_dt,
+                                hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && n > 0 && T_ <= 65535 * 32, "sigmoid_root: bad sizes");
+    ILM_REQUIRE(z_dt == ILM_DTYPE_F32 || z_dt == ILM_DTYPE_BF16, "sigmoid_root: unknown dtype %d", z_dt);
+    for (int t0 = 0; t0 < T_; t0 += 65535) {
+        const int rows = T_ - t0 < 65535 ? T_ - t0 : 65535;
+        dim3 grid((n + 255) / 256, rows);
+        if (z_dt == ILM_DTYPE_F32)
+            sigmoid_root_kernel<float><<<grid, 256, 0, stream>>>((float*)out + (size_t)t0 * out_stride,
+                                                                 (const float*)z + (size_t)t0 * in_stride, n, out_stride, in_stride, inv_tau);
+        else
+            sigmoid_root_kernel<bf16><<<grid, 256, 0, stream>>>((float*)out + (size_t)t0 * out_stride,
+                                                                (const bf16*)z + (size_t)t0 * in_stride, n, out_stride, in_stride, inv_tau);
+    }
+    ILM_LAUNCH_CHECK("sigmoid_root");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
 // Queries, keys and values of a linear-attention mixer made ready for the recurrence, as floats:
 // rows [q: heads*dk | k: heads*dk | v: heads*dv] of the fused projection -> the same layout in float, with an
 // activation on all three, then the first `rd` entries of each q and k head turned by the angle pos * freq[i]
@@ -265,14 +297,17 @@ __device__ __forceinline__ int sc_find(const int* __restrict__ seg_offsets, int 
     return (p >= 0 && p * piece < len) ? lo : -1;
 }
 
-template <int VC>   // VC: value columns a thread (the q and k a thread loads serve all of them)
+// CH: the decay comes per token, head and key channel (decay_c, rows of heads * dk floats dc_stride apart) and acts on the
+// state's rows: S_t = diag(a_t) S_(t-1) + ...
+template <int VC, bool CH = false>   // VC: value columns a thread (the q and k a thread loads serve all of them)
 __global__ void __launch_bounds__(256)
 decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__ q, const float* __restrict__ k,
                   int qk_stride, int q_div, const float* __restrict__ v, int v_stride,
                   const float* __restrict__ decay_h, const float* __restrict__ decay_t,
                   const float* __restrict__ kscale_t, const float* __restrict__ skip_h, float* __restrict__ pool,
                   const int* __restrict__ state_in, const int* __restrict__ state_out,
-                  const int* __restrict__ seg_offsets, int heads, int dk, int dv, int KP) {
+                  const int* __restrict__ seg_offsets, int heads, int dk, int dv, int KP,
+                  const float* __restrict__ decay_c = nullptr, int dc_stride = 0) {
     const int h = blockIdx.y, r = blockIdx.z;
     const int t0 = seg_offsets[r], t1 = seg_offsets[r + 1];
     if (t0 >= t1) return;
@@ -291,7 +326,7 @@ decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__
     const int qoff = (h / q_div) * dk;
     const float a_h = decay_h != nullptr ? decay_h[h] : 1.0f;
     const float skip = skip_h != nullptr ? skip_h[h] : 0.f;
-    float qn[SC_NK], kn[SC_NK], vn[VC], an, bn;
+    float qn[SC_NK], kn[SC_NK], vn[VC], an, bn, acn[CH ? SC_NK : 1];
 #define SC_LOAD(T_)                                                                              \
     {                                                                                            \
         const float* qr = q + (size_t)(T_) * qk_stride + qoff;                                   \
@@ -300,6 +335,7 @@ decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__
             const int ki = i * KP + kp;                                                          \
             qn[i] = ki < dk ? qr[ki] : 0.f;                                                      \
             kn[i] = ki < dk ? kr[ki] : 0.f;                                                      \
+            if (CH) acn[CH ? i : 0] = ki < dk ? decay_c[(size_t)(T_) * dc_stride + (size_t)h * dk + ki] : 0.f; \
         }                                                                                        \
         _Pragma("unroll") for (int c = 0; c < VC; ++c)                                           \
             vn[c] = vc0 + c < dv ? v[(size_t)(T_) * v_stride + (size_t)h * dv + vc0 + c] : 0.f;  \
@@ -308,12 +344,13 @@ decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__
     }
     SC_LOAD(t0)
     for (int t = t0; t < t1; ++t) {
-        float qc[SC_NK], kc[SC_NK], vcur[VC];
+        float qc[SC_NK], kc[SC_NK], vcur[VC], ac[SC_NK];
         const float a = an, b = bn;
 #pragma unroll
         for (int i = 0; i < SC_NK; ++i) {
             qc[i] = qn[i];
             kc[i] = kn[i] * b;
+            ac[i] = CH ? acn[CH ? i : 0] : a;
         }
 #pragma unroll
         for (int c = 0; c < VC; ++c) vcur[c] = vn[c];
@@ -324,7 +361,7 @@ decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__
             acc[c] = 0.f;
 #pragma unroll
             for (int i = 0; i < SC_NK; ++i) {
-                S[c][i] = fmaf(a, S[c][i], kc[i] * vcur[c]);
+                S[c][i] = fmaf(ac[i], S[c][i], kc[i] * vcur[c]);
                 acc[c] = fmaf(S[c][i], qc[i], acc[c]);
             }
         }
@@ -523,11 +560,15 @@ extern "C" int ilm_decay_scan(void* o, int o_stride, const void* q, const void* 
                               int v_stride, const void* decay_h, const void* decay_t, const void* kscale_t,
                               const void* skip_h, void* pool, const void* state_in, const void* state_out,
                               const void* seg_offsets, int R, int heads, int dk, int dv, int T_, int piece, void* ws_state,
-                              void* ws_decay, hipStream_t stream) {
+                              void* ws_decay, const void* decay_c, int dc_stride, hipStream_t stream) {
     ILM_REQUIRE(R > 0 && heads > 0 && dk > 0 && dv > 0 && T_ > 0, "decay_scan: bad sizes");
+    if (decay_c != nullptr) {
+        ILM_REQUIRE(decay_h == nullptr && decay_t == nullptr, "decay_scan: a decay per channel stands alone");
+        ILM_REQUIRE(piece == 0 && dc_stride >= heads * dk, "decay_scan: a decay per channel runs in one pass, rows of heads * dk");
+    }
     ILM_REQUIRE(dk <= SC_NK * 64, "decay_scan: %d state entries a column, at most %d", dk, SC_NK * 64);
     ILM_REQUIRE(q_div > 0 && heads % q_div == 0, "decay_scan: %d heads do not divide into groups of %d", heads, q_div);
-    ILM_REQUIRE((decay_h != nullptr) != (decay_t != nullptr), "decay_scan: a decay per head or per token, one of them");
+    ILM_REQUIRE(decay_c != nullptr || (decay_h != nullptr) != (decay_t != nullptr), "decay_scan: a decay per head or per token, one of them");
     ILM_REQUIRE(R <= 65535 && heads <= 65535, "decay_scan: too many requests or heads");
     ILM_REQUIRE(piece >= 0 && (piece == 0 || (ws_state != nullptr && ws_decay != nullptr)), "decay_scan: pieces need a workspace");
     int KP = 1;
@@ -539,6 +580,15 @@ extern "C" int ilm_decay_scan(void* o, int o_stride, const void* q, const void* 
     // four columns a thread where that still leaves two blocks a compute unit (long prompts in pieces, large batches):
     // a thread's loads of q and k then serve four columns; one column a thread where blocks are few (small batches)
     const int cus = ilm_num_cus();
+    if (piece == 0 && decay_c != nullptr) {
+        const int g4 = (dv + 4 * VT - 1) / (4 * VT);
+        if ((long)g4 * heads * R >= 2L * cus && dv >= 4)
+            decay_scan_kernel<4, true><<<dim3(g4, heads, R), 256, 0, stream>>>(SC_ARGS, (const float*)decay_c, dc_stride);
+        else
+            decay_scan_kernel<1, true><<<dim3((dv + VT - 1) / VT, heads, R), 256, 0, stream>>>(SC_ARGS, (const float*)decay_c, dc_stride);
+        ILM_LAUNCH_CHECK("decay_scan (decay per channel)");
+        return 0;
+    }
     if (piece == 0) {
         const int g4 = (dv + 4 * VT - 1) / (4 * VT);
         if ((long)g4 * heads * R >= 2L * cus && dv >= 4) decay_scan_kernel<4><<<dim3(g4, heads, R), 256, 0, stream>>>(SC_ARGS);

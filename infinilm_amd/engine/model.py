@@ -35,6 +35,10 @@ class CausalLM:
                                                                     hidden_size=spec.hidden_size, scale=spec.head.scale)), ctx)
         if spec.head.always_tied:
             self.output_head.tie(self.embedding.table)
+        self.run_vectors = None
+        if spec.run_vectors is not None:
+            self.run_vectors = torch.empty((int(spec.run_vectors[1]), spec.hidden_size), dtype=dtype, device=self.device)
+        self._keeps_embedding = any(r.start is not None and r.start.embedding != 0.0 for r in spec.order)
         # cache entry -> what its writer's mixer needs
         self.cache_needs: List = [None] * spec.num_cache_entries()
         for run in spec.order:
@@ -70,6 +74,8 @@ class CausalLM:
             out.update(b.named_parameters())
         for name, p in self.final_norm.named_parameters().items():
             out[join_name(self.spec.final_norm_name, name)] = p
+        if self.run_vectors is not None:
+            out[self.spec.run_vectors[0]] = Param(self.run_vectors)
         if not self.spec.head.always_tied:
             for name, p in self.output_head.named_parameters().items():
                 out[join_name(self.spec.head.name, name)] = p
@@ -95,7 +101,14 @@ class CausalLM:
         taps = batch.taps
         if taps is not None:
             taps["embed"] = stream.residual.clone()
+        # the embedding's output once more for the runs that add it again (the stream itself is summed into in place)
+        first = self.embedding.forward(batch.token_ids) if self._keeps_embedding else None
         for i, run in enumerate(self.spec.order):
+            if run.start is not None:
+                if run.start.embedding != 0.0:
+                    stream.push_more(first, run.start.embedding)
+                if run.start.vector_row is not None:
+                    stream.push_more(self.run_vectors[run.start.vector_row], 1.0)
             view = cache.view(run.cache, batch, run.writes_cache) if run.cache is not None else None
             self.blocks[run.layer].forward(stream, batch, view)
             if taps is not None:
@@ -104,6 +117,8 @@ class CausalLM:
                                    stream.pending_scale)
         if batch.num_wanted == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=self.device)
+        if stream.more:
+            stream.settle()
         if not batch.wants_all_rows:
             last = ResidualStream(kernels.gather_rows(stream.residual, batch.want_rows))
             if stream.pending is not None:

@@ -1071,10 +1071,11 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, dk
                pool: torch.Tensor, state_in: torch.Tensor, state_out: torch.Tensor, seg_offsets: torch.Tensor, segments: int,
                decay_h: Optional[torch.Tensor] = None, decay_t: Optional[torch.Tensor] = None,
                kscale_t: Optional[torch.Tensor] = None, skip_h: Optional[torch.Tensor] = None,
-               max_len: Optional[int] = None) -> torch.Tensor:
+               max_len: Optional[int] = None, decay_c: Optional[torch.Tensor] = None) -> torch.Tensor:
     """S_t = a_t S_(t-1) + (b_t k_t) v_t^T, o_t = S_t^T q_t + skip_h v_t for every head of every segment, token by token,
     all in float32.  q, k: [T, groups*dk] (views with one row stride; head h reads group h // (heads/groups)), v [T, heads*dv];
-    a per head (`decay_h` [heads]) or per token (`decay_t` [T, heads]); b `kscale_t` [T, heads] or absent.  `pool`
+    a per head (`decay_h` [heads]), per token (`decay_t` [T, heads]) or per token, head and key channel (`decay_c`
+    [T, heads*dk], float32 rows of one stride: S_t = diag(a_t) S_(t-1) + ..., always in one pass); b `kscale_t` [T, heads] or absent.  `pool`
     [rows, heads, dv, dk] holds the states: segment r starts from row state_in[r] and leaves its state in row state_out[r].
     `max_len`: a bound on the segments' lengths known on the host; from SCAN_PIECE_FROM tokens on, segments are cut
     into pieces of SCAN_PIECE tokens that run side by side (two passes and a combination of the pieces' states; the
@@ -1100,11 +1101,17 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, dk
                          (skip_h, (heads,), "skip_h")):
         if t is not None and (t.dtype != F32 or tuple(t.shape) != shape or not t.is_contiguous()):
             raise KernelError(f"{nm} must be contiguous float32 {shape}")
-    if (decay_h is None) == (decay_t is None):
+    if decay_c is not None:
+        _dev(decay_c)
+        _rows(decay_c, "decay_c")
+        if decay_h is not None or decay_t is not None or decay_c.dtype != F32 or decay_c.shape != (T, heads * dk):
+            raise KernelError(f"a decay per channel is float32 [{T}, {heads * dk}] and stands alone")
+    elif (decay_h is None) == (decay_t is None):
         raise KernelError("the recurrence takes a decay per head or per token, one of them")
     o = torch.empty((T, heads * dv), dtype=F32, device=v.device)
     piece, ws_state, ws_decay = 0, None, None
-    if SCAN_PIECE > 0 and max_len is not None and max_len >= SCAN_PIECE_FROM and T // SCAN_PIECE + int(segments) <= 65535:
+    if (decay_c is None and SCAN_PIECE > 0 and max_len is not None and max_len >= SCAN_PIECE_FROM
+            and T // SCAN_PIECE + int(segments) <= 65535):
         piece = SCAN_PIECE
         slots = T // piece + int(segments)
         ws_state = torch.empty((slots * heads * dv * dk,), dtype=F32, device=v.device)
@@ -1112,8 +1119,19 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, dk
     _run("ilm_decay_scan", o.data_ptr(), o.stride(0), q.data_ptr(), k.data_ptr(), q.stride(0), heads // groups, v.data_ptr(),
          v.stride(0), _ptr(decay_h), _ptr(decay_t), _ptr(kscale_t), _ptr(skip_h), pool.data_ptr(), state_in.data_ptr(),
          state_out.data_ptr(), seg_offsets.data_ptr(), int(segments), heads, dk, dv, T, piece, _ptr(ws_state), _ptr(ws_decay),
-         _stream())
+         _ptr(decay_c), decay_c.stride(0) if decay_c is not None else 0, _stream())
     return o
+
+
+def sigmoid_root(z: torch.Tensor, tau: float) -> torch.Tensor:
+    """float32 sigmoid(z)^(1/tau), element by element (the decays of a gated recurrence from their raw rows); z [T, n]
+    with dense rows."""
+    _dev(z)
+    _rows(z, "z")
+    T, n = z.shape
+    out = torch.empty((T, n), dtype=F32, device=z.device)
+    _run("ilm_sigmoid_root", out.data_ptr(), z.data_ptr(), T, n, out.stride(0), z.stride(0), 1.0 / float(tau), _dt(z), _stream())
+    return out
 
 
 def group_norm_gate(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, groups: int = 1,
@@ -1246,4 +1264,160 @@ def norm_add_norm(residual: torch.Tensor, branch: torch.Tensor, branch_weight: t
     _run("ilm_norm_add_norm", out.data_ptr(), residual.data_ptr(), branch.data_ptr(), branch_weight.data_ptr(), weight.data_ptr(),
          rows, H, float(alpha), float(branch_eps), float(eps), _dt(out), _dt(branch), _dt(branch_weight), _dt(weight), parts, pstride,
          _stream())
+    return out
+
+
+# ---- a sum of several addends into the residual stream + layer norm ---------------------------------
+LN_MAX_ADDENDS = 4   # (ilm_add_layernorm_max_addends())
+
+
+def add_layernorm(residual: torch.Tensor, addends, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float,
+                  out_dtype: torch.dtype) -> Optional[torch.Tensor]:
+    """residual += sum of scale * addend (in place, float32) over `addends` = [(tensor, scale), ...], then its layer norm
+    (x - mean) / sqrt(mean of squared deviations + eps) * weight + bias as out_dtype.  An addend is [rows, H] (float32 or
+    bfloat16), contiguous float32 parts [P, rows, H] that are summed in order, or one row [H] added to every row.
+    Without `weight` only the sum is done and None returned.  More addends than the kernel takes are summed by a call
+    of their own first."""
+    _dev(residual, weight, bias)
+    rows, H = residual.shape
+    if residual.dtype != F32 or not residual.is_contiguous():
+        raise KernelError("the residual stream is a contiguous float32 tensor")
+    addends = list(addends)
+    while len(addends) > LN_MAX_ADDENDS:
+        add_layernorm(residual, addends[:LN_MAX_ADDENDS], None, None, eps, out_dtype)
+        addends = addends[LN_MAX_ADDENDS:]
+    if weight is None and not addends:
+        return None
+    flat = []
+    for t, scale in addends:
+        _dev(t)
+        parts, pstride, rstride = 1, 0, H
+        if t.dim() == 1:
+            rstride = 0
+        elif t.dim() == 3:
+            parts, pstride = t.shape[0], t.stride(0)
+        if t.shape[-1] != H or (t.dim() > 1 and t.shape[-2] != rows) or not t.is_contiguous():
+            raise KernelError(f"an addend of shape {tuple(t.shape)} does not fit the residual stream {tuple(residual.shape)}")
+        flat += [t.data_ptr(), _dt(t), parts, pstride, rstride, float(scale)]
+    flat += [None, 0, 0, 0, 0, 0.0] * (LN_MAX_ADDENDS - len(addends))
+    out = None
+    if weight is not None:
+        if weight.shape != (H,) or not weight.is_contiguous() or (bias is not None and (bias.shape != (H,) or bias.dtype != weight.dtype
+                                                                                         or not bias.is_contiguous())):
+            raise KernelError(f"layer norm weight and bias must be [{H}] of one dtype")
+        out = torch.empty((rows, H), dtype=out_dtype, device=residual.device)
+    _run("ilm_add_layernorm", _ptr(out), residual.data_ptr(), _ptr(weight), _ptr(bias), rows, H, float(eps), _DT[out_dtype],
+         _dt(weight) if weight is not None else 0, len(addends), *flat, _stream())
+    return out
+
+
+# ---- attention with scores mixed over the heads ----------------------------------------------------
+def qkv_norm_rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, freq: Optional[torch.Tensor], q_weight: Optional[torch.Tensor],
+                          k_weight: Optional[torch.Tensor], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                          slots: Optional[torch.Tensor], nh: int, nkv: int, d: int, dn: int, dv: int, rd: int, v_norm: bool,
+                          eps: float) -> None:
+    """In the fused projection rows [T, (nh + 2 nkv) d]: every q and k head RMS-normed over its first `dn` entries times
+    `q_weight` / `k_weight` [dn] (None: no norm), then its entry pairs (2i, 2i + 1), i < rd / 2, turned by position x
+    freq[i]; every v head divided by its root mean square over its first `dv` entries (`v_norm`); k and v written to the
+    paged cache at `slots` (None: no write).  Entries of a head beyond those that count become zeros."""
+    _dev(qkv, positions, freq, q_weight, k_weight, k_cache, v_cache, slots)
+    _rows(qkv, "qkv")
+    _i32(positions, "positions")
+    T = qkv.shape[0]
+    if qkv.shape[1] != (nh + 2 * nkv) * d or positions.numel() != T:
+        raise KernelError(f"rows of {qkv.shape[1]} do not hold {nh} + 2 x {nkv} heads of {d}")
+    if rd and (freq is None or freq.dtype != F32 or freq.numel() != rd // 2 or not freq.is_contiguous()):
+        raise KernelError(f"frequencies must be float32 [{rd // 2}]")
+    for w in (q_weight, k_weight):
+        if w is not None and (w.shape != (dn,) or not w.is_contiguous() or w.dtype != (q_weight.dtype if q_weight is not None else w.dtype)):
+            raise KernelError(f"a query/key norm weight must be [{dn}]")
+    page = 1
+    if slots is not None:
+        _i32(slots, "slots")
+        if k_cache.dtype != qkv.dtype or slots.numel() != T:
+            raise KernelError("cache dtype or slots do not match the rows")
+        page = _check_cache(k_cache, v_cache, nkv, d)
+    _run("ilm_qkv_norm_rope_kvwrite", qkv.data_ptr(), positions.data_ptr(), _ptr(freq), _ptr(q_weight), _ptr(k_weight),
+         _ptr(k_cache) if slots is not None else None, _ptr(v_cache) if slots is not None else None, _ptr(slots), T, nh, nkv, d,
+         int(dn), int(dv), int(rd), int(bool(v_norm)), float(eps), page, qkv.stride(0), _dt(qkv),
+         _dt(q_weight) if q_weight is not None else _dt(qkv), _stream())
+
+
+def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                      seg_of_token: torch.Tensor, positions: torch.Tensor, nh: int, nkv: int, d: int, dv: int, scale: float,
+                      window: int = 0, mix: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Attention of every token over its request's cached keys (its last `window` positions, or all) where the scaled
+    scores of the heads are mixed before the softmax, s_h = sum_g mix[h, g] raw_g (`mix` float32 [nh, nh] or None),
+    and every head's denominator holds one more term exp(sink[h]) (`sink` float32 [nh] or None).  q, caches, block
+    tables as for `paged_attention`; `dv`: the entries of a value head that count.  Returns [T, nh*d]."""
+    _dev(q, k_cache, v_cache, block_tables, seg_of_token, positions, mix, sink)
+    _i32(block_tables, "block_tables")
+    _i32(seg_of_token, "seg_of_token")
+    _i32(positions, "positions")
+    T = q.shape[0]
+    if q.stride(1) != 1 or q.shape[1] < nh * d:
+        raise KernelError("q rows must be dense and hold all query heads")
+    if k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise KernelError(f"cache dtype {k_cache.dtype} differs from the activations' {q.dtype}")
+    page = _check_cache(k_cache, v_cache, nkv, d)
+    if seg_of_token.numel() != T or positions.numel() != T or block_tables.dim() != 2:
+        raise KernelError("per-token metadata does not match the number of tokens")
+    if mix is not None and (mix.dtype != F32 or tuple(mix.shape) != (nh, nh) or not mix.is_contiguous()):
+        raise KernelError(f"the heads' mixing matrix must be contiguous float32 [{nh}, {nh}]")
+    if sink is not None and (sink.dtype != F32 or tuple(sink.shape) != (nh,) or not sink.is_contiguous()):
+        raise KernelError(f"the denominators' extra terms must be contiguous float32 [{nh}]")
+    out = torch.empty((T, nh * d), dtype=q.dtype, device=q.device)
+    _run("ilm_attn_headmix", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
+         seg_of_token.data_ptr(), positions.data_ptr(), None, T, _ptr(mix), _ptr(sink), nh, nkv, d, int(dv), page,
+         block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window), _dt(q), _stream())
+    return out
+
+
+# ---- attention over latent rows -------------------------------------------------------------------
+def latent_prep(rows: torch.Tensor, qx: torch.Tensor, positions: torch.Tensor, freq: Optional[torch.Tensor], weight: torch.Tensor,
+                k_cache: torch.Tensor, v_cache: torch.Tensor, slots: Optional[torch.Tensor], heads: int, dn: int, dr: int, rank: int,
+                d: int, eps: float) -> None:
+    """From fused projection rows [q: heads (dn + dr) | down: rank + dr]: the latent c = RMS norm of down[:rank] times
+    `weight`, the last dr entries of `down` and of every query head turned in pairs (2i, 2i + 1) by position x freq[i];
+    key row [c | turned part | zeros] and value [c | zeros] into the one-head cache of head size d at `slots`; the
+    queries' turned parts (and zeros up to d) into qx [T, heads, d] from entry `rank` on."""
+    _dev(rows, qx, positions, freq, weight, k_cache, v_cache, slots)
+    _rows(rows, "rows")
+    _i32(positions, "positions")
+    T = rows.shape[0]
+    if tuple(qx.shape) != (T, heads, d) or not qx.is_contiguous() or qx.dtype != rows.dtype:
+        raise KernelError(f"the attention's query rows must be contiguous [{T}, {heads}, {d}] of the rows' dtype")
+    if rows.shape[1] != heads * (dn + dr) + rank + dr or weight.shape != (rank,) or not weight.is_contiguous():
+        raise KernelError("rows or norm weight do not fit the latent sizes")
+    if dr and (freq is None or freq.dtype != F32 or freq.numel() != dr // 2 or not freq.is_contiguous()):
+        raise KernelError(f"frequencies must be float32 [{dr // 2}]")
+    page = 1
+    if slots is not None:
+        _i32(slots, "slots")
+        if k_cache.dtype != rows.dtype or slots.numel() != T:
+            raise KernelError("cache dtype or slots do not match the rows")
+        page = _check_cache(k_cache, v_cache, 1, d)
+    _run("ilm_latent_prep", rows.data_ptr(), qx.data_ptr(), positions.data_ptr(), _ptr(freq), weight.data_ptr(),
+         _ptr(k_cache) if slots is not None else None, _ptr(v_cache) if slots is not None else None, _ptr(slots), T, heads, dn, dr,
+         rank, d, float(eps), page, rows.stride(0), _dt(rows), _dt(weight), _stream())
+
+
+HEAD_GEMM_LIBRARY_MIN_ROWS = 33   # rows from which the bfloat16 product per head goes to the vendor library
+
+
+def head_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, h, n] = sum_k x[t, h, k] w[h, k, n]: a product per head.  x [T, H, K] and out [T, H, N] are views with
+    a dense last axis; w [H, K, N] is a view one of whose last two axes is dense.  Float sums."""
+    _dev(x, w, out)
+    T, H, K = x.shape
+    N = w.shape[2]
+    if tuple(w.shape) != (H, K, N) or tuple(out.shape) != (T, H, N) or x.stride(2) != 1 or out.stride(2) != 1 \
+            or x.dtype != w.dtype or (w.stride(1) != 1 and w.stride(2) != 1):
+        raise KernelError(f"a product per head of {tuple(x.shape)} x {tuple(w.shape)} -> {tuple(out.shape)} does not fit")
+    if x.dtype == BF16 and out.dtype == BF16 and T >= HEAD_GEMM_LIBRARY_MIN_ROWS and USE_LIBRARY_GEMM and not FORCE_BASIC:
+        with _timed("library_gemm"):
+            out.copy_(torch.bmm(x.transpose(0, 1), w).transpose(0, 1))
+        return out
+    _run("ilm_head_gemm", out.data_ptr(), x.data_ptr(), w.data_ptr(), T, N, K, H, x.stride(0), x.stride(1), w.stride(0),
+         w.stride(1), w.stride(2), out.stride(0), out.stride(1), _dt(x), _dt(out), _stream())
     return out

@@ -15,7 +15,7 @@ import torch
 from .. import kernels
 from ..cache.needs import PagedKV
 from ..config.spec import PartSpec
-from .base import BuildContext, Mixer, Param
+from .base import BuildContext, Mixer, Param, join_name
 from .linear import FusedLinear, Linear
 from .registry import build_position_encoding, register_mixer
 
@@ -30,13 +30,19 @@ class GQAttention(Mixer):
     The cache and the attention kernels know one head size: query/key heads and value heads of different sizes (or
     of a size that is no multiple of 16) are filled up with zeros to the next multiple of 16 that holds both, in the
     projections' weights: zero entries add nothing to a score, and the output entries they make meet zero columns
-    of the output projection."""
+    of the output projection.
+
+    `head_mix`: the scaled scores are mixed over the heads before the softmax, s_h = sum_g M[h, g] raw_g, with a tensor
+    M [heads, heads]; `sink`: every head's softmax denominator holds one more term exp(sink_h), a tensor [heads] with no
+    key and no value.  Both are float32 whatever the activations' dtype; `mix_names` are their tensor names.
+    `position_prefix`: the sub-name under which the position encoding's own tensors lie ("": directly under the mixer's)."""
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, qkv_bias: bool,
                  out_bias: bool, scale: float, window: int, position: PartSpec, ctx: BuildContext,
                  value_dim: Optional[int] = None, softcap: float = 0.0,
                  names: Sequence[str] = ("q_proj", "k_proj", "v_proj", "o_proj"), suffix: str = "weight",
-                 whole_output: bool = False):
+                 whole_output: bool = False, head_mix: bool = False, sink: bool = False,
+                 mix_names: Sequence[str] = ("head_mix", "sink"), position_prefix: str = "position", bias_suffix: str = "bias"):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads do not divide into {num_kv_heads} groups")
         self.nh, self.nkv = int(num_heads), int(num_kv_heads)
@@ -49,11 +55,15 @@ class GQAttention(Mixer):
         self.whole_output = bool(whole_output)
         qn, kn, vn, on = names
         self.qkv = FusedLinear(hidden_size, [self.nh * self.d, self.nkv * self.d, self.nkv * self.d], [qn, kn, vn],
-                               qkv_bias, ctx, suffix=suffix,
+                               qkv_bias, ctx, suffix=suffix, bias_suffix=bias_suffix,
                                out_heads=[(self.nh, self.dn, self.d), (self.nkv, self.dn, self.d), (self.nkv, self.dv, self.d)])
-        self.o_proj = Linear(self.nh * self.d, hidden_size, on, out_bias, ctx, suffix=suffix,
+        self.o_proj = Linear(self.nh * self.d, hidden_size, on, out_bias, ctx, suffix=suffix, bias_suffix=bias_suffix,
                              in_heads=(self.nh, self.dv, self.d))
         self.position = build_position_encoding(position, ctx)
+        self.position_prefix = position_prefix
+        self.mix_names = tuple(mix_names)
+        self.head_mix = torch.empty((self.nh, self.nh), dtype=torch.float32, device=ctx.device) if head_mix else None
+        self.sink = torch.empty((self.nh,), dtype=torch.float32, device=ctx.device) if sink else None
         if getattr(self.position, "head_dim", self.d) not in (0, self.d):
             raise ValueError(f"the position encoding is made for heads of {self.position.head_dim}, the mixer's have {self.d}")
 
@@ -61,7 +71,11 @@ class GQAttention(Mixer):
         out = dict(self.qkv.named_parameters())
         out.update(self.o_proj.named_parameters())
         for name, p in self.position.named_parameters().items():   # an encoding may bring tensors of its own
-            out[f"position.{name}"] = p
+            out[join_name(self.position_prefix, name)] = p
+        if self.head_mix is not None:
+            out[self.mix_names[0]] = Param(self.head_mix)
+        if self.sink is not None:
+            out[self.mix_names[1]] = Param(self.sink)
         return out
 
     def cache_need(self):
@@ -85,11 +99,22 @@ class GQAttention(Mixer):
             pe.encode_and_store(qkv, batch, cache_view, self.nh, self.nkv, self.d)
             if batch.taps is not None:
                 batch.taps.setdefault("qkv_rotated", []).append(qkv.clone())
-        o = kernels.paged_attention(qkv, cache_view.k, cache_view.v, cache_view.block_tables, batch.seg_of_token,
-                                    batch.positions, self.nh, self.nkv, self.d, self.scale, self.window,
-                                    batch.max_total_len, batch.att_tiles, batch.att_single_rows, softcap=self.softcap)
+        if self.head_mix is not None or self.sink is not None:
+            if self.softcap:
+                raise ValueError("scores mixed over the heads take no cap")
+            o = kernels.headmix_attention(qkv, cache_view.k, cache_view.v, cache_view.block_tables, batch.seg_of_token,
+                                          batch.positions, self.nh, self.nkv, self.d, self.dv, self.scale, self.window,
+                                          mix=self.head_mix, sink=self.sink)
+        else:
+            o = self._plain_attention(qkv, batch, cache_view)
         if tail is not None:   # the output projection adds into the residual stream itself, where its kernel can
             deferred = self.o_proj.forward_tail(o, tail)
             if deferred is not None:
                 return deferred
         return self.o_proj.forward(o, allow_parts=not self.whole_output)
+
+    def _plain_attention(self, qkv, batch, cache_view):
+        o = kernels.paged_attention(qkv, cache_view.k, cache_view.v, cache_view.block_tables, batch.seg_of_token,
+                                    batch.positions, self.nh, self.nkv, self.d, self.scale, self.window,
+                                    batch.max_total_len, batch.att_tiles, batch.att_single_rows, softcap=self.softcap)
+        return o

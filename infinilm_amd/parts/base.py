@@ -81,6 +81,15 @@ class ResidualStream:
         # a branch that is still to be normed by `pending_norm` before it is added (an arrangement with a norm on every
         # sublayer's output): a norm that knows how does both in its own kernel, anybody else calls `settle()` first
         self.pending_norm = None
+        # further addends (tensor, scale) that are due to the stream beside `pending`: a second branch that read the same
+        # norm's output, a copy of the embedding's output, one row for all tokens.  A norm that knows how sums them in its
+        # own kernel; anybody else calls `settle()` first
+        self.more: list = []
+
+    def push_more(self, addend: torch.Tensor, scale: float = 1.0) -> None:
+        """`addend` ([T, hidden], float32 parts [P, T, hidden], or one row [hidden] for every token) times `scale` joins
+        the stream when it is next read."""
+        self.more.append((addend, float(scale)))
 
     def push(self, branch: torch.Tensor, scale: float) -> None:
         if self.pending is not None:
@@ -99,6 +108,10 @@ class ResidualStream:
         if self.pending_norm is not None:
             norm, self.pending_norm = self.pending_norm, None
             self.pending = norm.apply(self.pending)
+        if self.more:
+            from .. import kernels
+            more, self.more = self.more, []
+            kernels.add_layernorm(self.residual, more, None, None, 0.0, torch.float32)
 
 
 @dataclass

@@ -111,6 +111,43 @@ class SandwichNormBlock:
             stream.push_normed(y, self.norm2b, self.residual_scale)
 
 
+@register_arrangement("parallel_residual")
+class ParallelResidualBlock:
+    """x += s * (mixer(h) + ffn(h)) with h = norm1(x): one norm, and both sublayers read its output.  A layer may have no
+    feed-forward.  Both outputs are left with the stream and summed into it inside the next norm's kernel."""
+
+    def __init__(self, spec: LayerSpec, ctx: BuildContext):
+        self.spec = spec
+        self.slots = tuple(s for s in ("norm1", "mixer", "ffn") if s in spec.parts)
+        if not {"norm1", "mixer"} <= set(self.slots):
+            raise ValueError(f"layer {spec.prefix}: a parallel layer has norm1, mixer and, if any, ffn")
+        self.norm1 = build_norm(spec.parts["norm1"], ctx)
+        self.mixer = build_mixer(spec.parts["mixer"], ctx)
+        self.ffn = build_feed_forward(spec.parts["ffn"], ctx) if "ffn" in self.slots else None
+        self.residual_scale = float(spec.residual_scale)
+
+    def named_parameters(self) -> Dict[str, Param]:
+        out: Dict[str, Param] = {}
+        for slot in self.slots:
+            for name, p in getattr(self, slot).named_parameters().items():
+                out[join_name(self.spec.prefix, self.spec.names[slot], name)] = p
+        return out
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    @property
+    def records_mixed_steps(self) -> bool:
+        return bool(getattr(self.mixer, "records_mixed_steps", False)
+                    and (self.ffn is None or getattr(self.ffn, "records_mixed_steps", False)))
+
+    def forward(self, stream: ResidualStream, batch, cache_view) -> None:
+        h = self.norm1.forward(stream)
+        stream.push(self.mixer.forward(h, batch, cache_view), self.residual_scale)
+        if self.ffn is not None:
+            stream.push_more(self.ffn.forward(h, batch), self.residual_scale)
+
+
 def build_block(spec: LayerSpec, ctx: BuildContext):
     try:
         cls = ARRANGEMENTS[spec.arrangement]

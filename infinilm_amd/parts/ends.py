@@ -55,14 +55,15 @@ class ScaledLookup(Embedding):
 class LinearHead(OutputHead):
     """logits = scale * x W^T, float32."""
 
-    def __init__(self, vocab_size: int, hidden_size: int, scale: float, ctx: BuildContext):
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float, ctx: BuildContext, param_name: str = "weight"):
         self.scale = float(scale)
+        self.param_name = param_name    # "": the matrix lies under the head's own name in a checkpoint
         self.weight: Optional[torch.Tensor] = torch.empty((int(vocab_size), int(hidden_size)), dtype=ctx.dtype,
                                                           device=ctx.device)
         self.tied = False
 
     def named_parameters(self) -> Dict[str, Param]:
-        return {"weight": Param(self.weight)}
+        return {self.param_name: Param(self.weight)}
 
     def tie(self, table: torch.Tensor) -> None:
         if tuple(table.shape) != tuple(self.weight.shape):

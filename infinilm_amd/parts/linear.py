@@ -26,8 +26,9 @@ class FusedLinear:
 
     def __init__(self, in_features: int, out_sizes: Sequence[int], names: Sequence[str], bias: bool,
                  ctx: BuildContext, suffix: str = "weight", out_heads: Optional[Sequence] = None,
-                 in_heads: Optional[tuple] = None):
+                 in_heads: Optional[tuple] = None, bias_suffix: str = "bias"):
         self.in_features = int(in_features)
+        self.bias_suffix = bias_suffix      # a bias's name is `names[i]` + "." + bias_suffix
         self.out_sizes = [int(s) for s in out_sizes]
         self.names = list(names)
         self.suffix = suffix
@@ -55,14 +56,14 @@ class FusedLinear:
                 heads, real, pad = oh
                 out[join_name(name, self.suffix)] = Param(w.view(heads, pad, self.in_features)[:, :real], shape=(heads * real, self.in_features))
                 if b is not None:
-                    out[join_name(name, "bias")] = Param(b.view(heads, pad)[:, :real], shape=(heads * real,))
+                    out[join_name(name, self.bias_suffix)] = Param(b.view(heads, pad)[:, :real], shape=(heads * real,))
             elif self.in_heads is not None:
                 heads, real, pad = self.in_heads
                 out[join_name(name, self.suffix)] = Param(w.view(size, heads, pad)[:, :, :real], shape=(size, heads * real))
             else:
                 out[join_name(name, self.suffix)] = Param(w)
                 if b is not None:
-                    out[join_name(name, "bias")] = Param(b)
+                    out[join_name(name, self.bias_suffix)] = Param(b)
             row += size
         return out
 
@@ -95,5 +96,5 @@ class FusedLinear:
 
 class Linear(FusedLinear):
     def __init__(self, in_features: int, out_features: int, name: str, bias: bool, ctx: BuildContext,
-                 suffix: str = "weight", in_heads: Optional[tuple] = None):
-        super().__init__(in_features, [out_features], [name], bias, ctx, suffix=suffix, in_heads=in_heads)
+                 suffix: str = "weight", in_heads: Optional[tuple] = None, bias_suffix: str = "bias"):
+        super().__init__(in_features, [out_features], [name], bias, ctx, suffix=suffix, in_heads=in_heads, bias_suffix=bias_suffix)

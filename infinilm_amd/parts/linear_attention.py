@@ -97,3 +97,66 @@ class LightningAttention(DecayLinearAttention):
     def __init__(self, hidden_size, heads, key_dim, value_dim, decay, eps, ctx, **names):
         super().__init__(hidden_size, heads, key_dim, value_dim, decay, eps, ctx, activation="silu", rotary=None,
                          k_scale=1.0, norm="all", norm_weight=True, gate_act="sigmoid", **names)
+
+
+@register_mixer("gated_linear_attention")
+class GatedLinearAttention(Mixer):
+    """Linear attention whose state decays per key channel by a gate computed from the input:
+
+      q = W_q h / sqrt(dk), k = W_k h [heads, dk], v = W_v h [heads, dv]
+      alpha = sigmoid(W_a2 (W_a1 h) + b)^(1/tau)  [heads, dk]      a low-rank pair of projections
+      S_t = diag(alpha_t) S_(t-1) + k_t v_t^T,  o_t = S_t^T q_t      per head, S [dk, dv] starts at zero
+      o RMS-normed per head over dv with a weight [dv] shared by the heads, times silu(W_g h), then W_o.
+
+    The 1/sqrt(dk) is applied to k instead of q (the state is linear in k).  Decays, state, norm and gate are float32
+    whatever the activations' dtype; the state lives in a row of the cache manager's pool, [heads, dv, dk].  The low rank
+    is the number of rows of W_a1."""
+    records_mixed_steps = True
+
+    def __init__(self, hidden_size: int, heads: int, key_dim: int, value_dim: int, decay_rank: int, tau: float, eps: float,
+                 ctx: BuildContext, names: Sequence[str] = ("q", "k", "v", "g", "a1", "a2", "o", "norm"), suffix: str = "",
+                 bias_suffix: str = "bias", whole_output: bool = False):
+        self.H, self.dk, self.dv, self.low = int(heads), int(key_dim), int(value_dim), int(decay_rank)
+        if self.dk > kernels.SCAN_MAX_KEY_DIM:
+            raise ValueError(f"key size {self.dk} is above the recurrence kernel's {kernels.SCAN_MAX_KEY_DIM}")
+        if tau <= 0:
+            raise ValueError(f"tau {tau} must be positive")
+        self.tau, self.eps = float(tau), float(eps)
+        self.whole_output = bool(whole_output)
+        self.dtype = ctx.dtype
+        qn, kn, vn, gn, a1n, a2n, on, self.norm_name = names
+        H, dk, dv = self.H, self.dk, self.dv
+        self.proj = FusedLinear(hidden_size, [H * dk, H * dk, H * dv, H * dv, self.low], [qn, kn, vn, gn, a1n], False, ctx, suffix=suffix)
+        self.a2 = Linear(self.low, H * dk, a2n, True, ctx, suffix=suffix, bias_suffix=bias_suffix)
+        self.o_proj = Linear(H * dv, hidden_size, on, False, ctx, suffix=suffix)
+        self.norm_w = torch.empty((dv,), dtype=ctx.dtype, device=ctx.device)
+        self._norm_all = None     # (version, the weight once for every head)
+
+    def named_parameters(self) -> Dict[str, Param]:
+        out = dict(self.proj.named_parameters())
+        out.update(self.a2.named_parameters())
+        out.update(self.o_proj.named_parameters())
+        out[self.norm_name] = Param(self.norm_w, neutral=1.0)
+        return out
+
+    def cache_need(self):
+        return FixedState((self.H, self.dv, self.dk), torch.float32)
+
+    def _norm_weight(self) -> torch.Tensor:
+        held = self._norm_all
+        if held is None or held[0] != (self.norm_w._version, self.norm_w.data_ptr()):
+            held = self._norm_all = ((self.norm_w._version, self.norm_w.data_ptr()), self.norm_w.repeat(self.H).contiguous())
+        return held[1]
+
+    def forward(self, x, batch, view):
+        H, dk, dv = self.H, self.dk, self.dv
+        rows = self.proj.forward(x)                                    # [T, q | k | v | g | low]
+        g0 = 2 * H * dk + H * dv
+        z = self.a2.forward(rows[:, g0 + H * dv:], out_dtype=torch.float32)          # [T, heads * dk]
+        alpha = kernels.sigmoid_root(z, self.tau)
+        f = kernels.linear_attention_inputs(rows, None, None, H, dk, dv, 0, "none", float(dk) ** -0.5)
+        o = kernels.decay_scan(f[:, :H * dk], f[:, H * dk:2 * H * dk], f[:, 2 * H * dk:], H, dk, dv, H, view.pool,
+                               view.state_in, view.state_out, batch.seg_offsets, view.state_in.numel(), decay_c=alpha)
+        y = kernels.group_norm_gate(o, self._norm_weight(), self.eps, H, gate=rows[:, g0:g0 + H * dv], gate_act="silu",
+                                    out_dtype=self.dtype)
+        return self.o_proj.forward(y, allow_parts=not self.whole_output)

@@ -46,6 +46,8 @@ class RMSNorm(Norm):
 
     def forward(self, stream: ResidualStream, frag: bool = False):
         """`frag`: the consumer takes its rows in fragment order (`kernels.FragRows`)."""
+        if stream.more:
+            stream.settle()
         post = stream.pending_norm
         if post is not None and not frag and isinstance(post, RMSNorm):
             # the branch's own norm, the sum and this norm in one kernel
@@ -58,4 +60,33 @@ class RMSNorm(Norm):
                                 self.dtype, frag=frag)
         stream.pending = None
         stream.pending_scale = 1.0
+        return x
+
+
+@register_norm("layernorm")
+class LayerNorm(Norm):
+    """(x - mean) / sqrt(mean of squared deviations + eps) * weight + bias, fused with the sums that are due to the residual
+    stream: the pending branch and every further addend (`ResidualStream.more`) are added in the same kernel.
+    `param_name` / `bias_name`: the tensors' names under the norm's own name ("": the norm's name itself)."""
+
+    def __init__(self, size: int, eps: float, ctx: BuildContext, bias: bool = True, param_name: str = "weight",
+                 bias_name: str = "bias"):
+        self.size, self.eps, self.dtype = int(size), float(eps), ctx.dtype
+        self.param_name, self.bias_name = param_name, bias_name
+        self.weight = torch.empty((self.size,), dtype=ctx.dtype, device=ctx.device)
+        self.bias = torch.empty((self.size,), dtype=ctx.dtype, device=ctx.device) if bias else None
+
+    def named_parameters(self) -> Dict[str, Param]:
+        out = {self.param_name: Param(self.weight, neutral=1.0)}
+        if self.bias is not None:
+            out[self.bias_name] = Param(self.bias)
+        return out
+
+    def forward(self, stream: ResidualStream, frag: bool = False):
+        if stream.pending_norm is not None:
+            norm, stream.pending_norm = stream.pending_norm, None
+            stream.pending = norm.apply(stream.pending)
+        addends = ([(stream.pending, stream.pending_scale)] if stream.pending is not None else []) + stream.more
+        x = kernels.add_layernorm(stream.residual, addends, self.weight, self.bias, self.eps, self.dtype)
+        stream.pending, stream.pending_scale, stream.more = None, 1.0, []
         return x

@@ -173,3 +173,46 @@ class NoPositionEncoding(RotaryEmbedding):
 
     def project_encode_store(self, x, proj, batch, view, nh, nkv, d):
         return None
+
+
+def pair_frequencies(dims: int, base: float, device) -> Optional[torch.Tensor]:
+    """float32 [dims / 2]: base^(-2i/dims), formed in float64 (None for no dims)."""
+    if dims <= 0:
+        return None
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims).to(torch.float32).to(device)
+
+
+@register_position_encoding("normed_pair_rotary")
+class NormedPairRotary(PositionEncoding):
+    """Queries and keys normed per head, then turned in neighbouring pairs; values of unit size:
+
+      q <- q / sqrt(mean(q^2) + eps) * w_q,  k likewise with w_k          per head over its `dim` entries, the weights
+                                                                           [dim] shared by the heads (`qk_norm`)
+      (x_2i, x_2i+1) <- (x_2i cos a - x_2i+1 sin a, x_2i+1 cos a + x_2i sin a),  a = p * theta^(-2i / rotary_dim),
+                                                                           i < rotary_dim / 2, for q and k at position p
+      v <- v / sqrt(mean(v^2) + eps)                                       per head over its `value_dim` entries (`v_norm`)
+
+    One kernel does all of it and writes k and v into the cache.  The angle is formed in float32 from the position in
+    the kernel (no table, so no bound on positions).  `names`: the two weights' tensor names."""
+    head_dim = 0    # any size the mixer runs: the entries beyond `dim` / `value_dim` are zeros
+
+    def __init__(self, dim: int, value_dim: int, rotary_dim: int, theta: float, eps: float, ctx: BuildContext,
+                 qk_norm: bool = True, v_norm: bool = False, names=("q_norm", "k_norm")):
+        self.dim, self.value_dim, self.rotary_dim = int(dim), int(value_dim), int(rotary_dim)
+        if self.rotary_dim % 2 or not 0 <= self.rotary_dim <= self.dim:
+            raise ValueError(f"rotary_dim {rotary_dim} must be even and at most the head size {dim}")
+        self.eps, self.v_norm, self.names = float(eps), bool(v_norm), tuple(names)
+        self.freq = pair_frequencies(self.rotary_dim, theta, ctx.device)
+        self.q_weight = torch.empty((self.dim,), dtype=ctx.dtype, device=ctx.device) if qk_norm else None
+        self.k_weight = torch.empty((self.dim,), dtype=ctx.dtype, device=ctx.device) if qk_norm else None
+
+    def named_parameters(self):
+        if self.q_weight is None:
+            return {}
+        from .base import Param
+        return {self.names[0]: Param(self.q_weight, neutral=1.0), self.names[1]: Param(self.k_weight, neutral=1.0)}
+
+    def encode_and_store(self, qkv, batch, view, nh, nkv, d):
+        kernels.qkv_norm_rope_kvwrite(qkv, batch.positions, self.freq, self.q_weight, self.k_weight, view.k, view.v, view.slots,
+                                      nh, nkv, d, self.dim, self.value_dim, self.rotary_dim, self.v_norm, self.eps)

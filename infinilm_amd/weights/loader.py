@@ -53,6 +53,22 @@ def weight_files(model_dir: str) -> List[str]:
     return files
 
 
+def checkpoint_shapes(model_dir: str) -> dict:
+    """{tensor name: shape} of the folder's safetensors, read from the files' headers alone (8 bytes of length,
+    little-endian, then that many bytes of JSON)."""
+    out = {}
+    for path in weight_files(model_dir):
+        with open(path, "rb") as fh:
+            n = int.from_bytes(fh.read(8), "little")
+            if not 0 < n <= 1 << 30:
+                raise ValueError(f"{path}: not a safetensors file")
+            header = json.loads(fh.read(n))
+        for name, rec in header.items():
+            if name != "__metadata__":
+                out[name] = tuple(rec["shape"])
+    return out
+
+
 def iter_tensors(model_dir: str) -> Iterator[Tuple[str, torch.Tensor]]:
     from safetensors import safe_open
 
