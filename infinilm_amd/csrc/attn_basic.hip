@@ -22,12 +22,13 @@
 
 // (M, L, ACC) <- fold of (M, L, ACC) and a chunk's (m, l, acc); explicit multiply-adds, so that the two
 // launch shapes round alike
-__device__ __forceinline__ void ab_fold(float& M, float& L, float (&ACC)[4], float m, float l, const float (&acc)[4]) {
+template <int NA>
+__device__ __forceinline__ void ab_fold(float& M, float& L, float (&ACC)[NA], float m, float l, const float (&acc)[NA]) {
     const float Mn = fmaxf(M, m);
     const float a = expf(M - Mn), b = expf(m - Mn);
     L = fmaf(L, a, l * b);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) ACC[i] = fmaf(ACC[i], a, acc[i] * b);
+    for (int i = 0; i < NA; ++i) ACC[i] = fmaf(ACC[i], a, acc[i] * b);
     M = Mn;
 }
 
@@ -48,7 +49,7 @@ __device__ __forceinline__ void load4(const bf16* p, float* v) {
         const int pg = bt[key / page];                                                         \
         const T* vcol = vc + ((size_t)pg * nkv + kvh) * d * page + (key % page);               \
         const float w = ps[J_];                                                                \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                        \
+        _Pragma("unroll") for (int i = 0; i < NA; ++i) {                                       \
             const int dim = lane + 64 * i;                                                     \
             if (dim < d) acc[i] = fmaf(w, to_f32(vcol[(size_t)dim * page]), acc[i]);           \
         }                                                                                      \
@@ -57,7 +58,8 @@ __device__ __forceinline__ void load4(const bf16* p, float* v) {
 // VEC: the head size and the page size are multiples of 4 and the tensors 16 bytes aligned: 16-byte loads.
 // ws == nullptr: gridDim.z == 1, the wave walks all chunks.  Else blockIdx.z is the chunk (absolute
 // index) and the partial result goes to ws[((t * nh + h) * gridDim.z + chunk) * (d + 2)]: d outputs, m, l.
-template <typename T, bool VEC>
+// NA: 64 * NA is the largest head size (4 for heads up to 256, 16 up to 1024).
+template <typename T, bool VEC, int NA>
 __global__ void __launch_bounds__(64)
 attn_basic_kernel(T* __restrict__ out, float* __restrict__ ws, const T* __restrict__ q, const T* __restrict__ kc,
                   const T* __restrict__ vc, const int* __restrict__ block_tables,
@@ -81,12 +83,16 @@ attn_basic_kernel(T* __restrict__ out, float* __restrict__ ws, const T* __restri
     __syncthreads();
 
     float M = -INFINITY, L = 0.f;
-    float ACC[4] = {0.f, 0.f, 0.f, 0.f};
+    float ACC[NA];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) ACC[i] = 0.f;
     for (int c = c_first; c <= c_last; ++c) {
         const int k_lo = lo > c * AB_CHUNK ? lo : c * AB_CHUNK;
         const int k_hi = p < c * AB_CHUNK + AB_CHUNK - 1 ? p : c * AB_CHUNK + AB_CHUNK - 1;
         float m = -INFINITY, l = 0.f;
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        float acc[NA];
+#pragma unroll
+        for (int i = 0; i < NA; ++i) acc[i] = 0.f;
         for (int tile = k_lo >> 6; tile <= (k_hi >> 6); ++tile) {
             const int kidx = (tile << 6) + lane;
             const bool valid = kidx >= k_lo && kidx <= k_hi;
@@ -115,7 +121,7 @@ attn_basic_kernel(T* __restrict__ out, float* __restrict__ ws, const T* __restri
             ps[lane] = pj;
             __syncthreads();
 #pragma unroll
-            for (int i = 0; i < 4; ++i) acc[i] *= corr;
+            for (int i = 0; i < NA; ++i) acc[i] *= corr;
             const int j0 = (k_lo > (tile << 6)) ? k_lo - (tile << 6) : 0;
             const int j1 = (k_hi - (tile << 6) < 63) ? k_hi - (tile << 6) : 63;
             int j = j0;
@@ -129,7 +135,7 @@ attn_basic_kernel(T* __restrict__ out, float* __restrict__ ws, const T* __restri
                     const T* vcol = vc + ((size_t)pg * nkv + kvh) * d * page + (key % page);
                     const float w0 = ps[j], w1 = ps[j + 1], w2 = ps[j + 2], w3 = ps[j + 3];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
+                    for (int i = 0; i < NA; ++i) {
                         const int dim = lane + 64 * i;
                         if (dim < d) {
                             float vv[4];
@@ -149,7 +155,7 @@ attn_basic_kernel(T* __restrict__ out, float* __restrict__ ws, const T* __restri
         if (ws != nullptr) {
             float* dst = ws + (((size_t)t * nh + h) * gridDim.z + c) * (d + 2);
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < NA; ++i) {
                 const int dim = lane + 64 * i;
                 if (dim < d) dst[dim] = acc[i];
             }
@@ -159,19 +165,19 @@ attn_basic_kernel(T* __restrict__ out, float* __restrict__ ws, const T* __restri
             }
             return;
         }
-        ab_fold(M, L, ACC, m, l, acc);
+        ab_fold<NA>(M, L, ACC, m, l, acc);
     }
     T* orow = out + (size_t)t * out_stride + (size_t)h * d;
     const float inv = 1.0f / L;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NA; ++i) {
         const int dim = lane + 64 * i;
         if (dim < d) orow[dim] = from_f32<T>(ACC[i] * inv);
     }
 }
 
 // Folds the chunks' partial results of one (token, head), in ascending order, as the one-wave shape does.
-template <typename T>
+template <typename T, int NA>
 __global__ void __launch_bounds__(64)
 attn_basic_fold_kernel(T* __restrict__ out, const float* __restrict__ ws, const int* __restrict__ pos, int nh, int d,
                        int nchunks, int out_stride, int window) {
@@ -186,21 +192,23 @@ attn_basic_fold_kernel(T* __restrict__ out, const float* __restrict__ ws, const 
         return;
     }
     float M = -INFINITY, L = 0.f;
-    float ACC[4] = {0.f, 0.f, 0.f, 0.f};
+    float ACC[NA];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) ACC[i] = 0.f;
     for (int c = lo / AB_CHUNK; c <= p / AB_CHUNK; ++c) {
         const float* src = ws + (((size_t)t * nh + h) * nchunks + c) * (d + 2);
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        float acc[NA];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < NA; ++i) {
             const int dim = lane + 64 * i;
-            if (dim < d) acc[i] = src[dim];
+            acc[i] = dim < d ? src[dim] : 0.f;
         }
-        ab_fold(M, L, ACC, src[d], src[d + 1], acc);
+        ab_fold<NA>(M, L, ACC, src[d], src[d + 1], acc);
     }
     T* orow = out + (size_t)t * out_stride + (size_t)h * d;
     const float inv = 1.0f / L;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int i = 0; i < NA; ++i) {
         const int dim = lane + 64 * i;
         if (dim < d) orow[dim] = from_f32<T>(ACC[i] * inv);
     }
@@ -217,7 +225,7 @@ extern "C" int ilm_attn_basic(void* out, void* ws, int nchunks, const void* q, c
                               hipStream_t stream) {
     ILM_REQUIRE(T_ > 0 && nh > 0 && nkv > 0 && d > 0 && page > 0 && max_blocks > 0, "attn_basic: bad sizes");
     ILM_REQUIRE(nh % nkv == 0, "attn_basic: %d query heads do not divide into %d groups", nh, nkv);
-    ILM_REQUIRE(d <= 256, "attn_basic: head size %d above 256", d);
+    ILM_REQUIRE(d <= 1024, "attn_basic: head size %d above 1024", d);
     ILM_REQUIRE(nh <= 65535, "attn_basic: too many heads");
     ILM_REQUIRE(ws == nullptr || (nchunks >= 1 && nchunks <= 65535), "attn_basic: %d chunks", nchunks);
     ILM_REQUIRE(dtype == ILM_DTYPE_F32 || dtype == ILM_DTYPE_BF16, "attn_basic: unknown dtype %d", dtype);
@@ -225,24 +233,30 @@ extern "C" int ilm_attn_basic(void* out, void* ws, int nchunks, const void* q, c
     const size_t shm = (size_t)(d + 64) * sizeof(float);
     const bool vec = d % 4 == 0 && page % 4 == 0 && ((uintptr_t)kc & 15) == 0 && ((uintptr_t)vc & 15) == 0;
 #define AB_LAUNCH(T_, VEC_)                                                                                             \
-    attn_basic_kernel<T_, VEC_><<<grid, 64, shm, stream>>>(                                                             \
+    if (d <= 256) AB_LAUNCH_N(T_, VEC_, 4); else AB_LAUNCH_N(T_, VEC_, 16)
+#define AB_LAUNCH_N(T_, VEC_, NA_)                                                                                      \
+    attn_basic_kernel<T_, VEC_, NA_><<<grid, 64, shm, stream>>>(                                                        \
         (T_*)out, (float*)ws, (const T_*)q, (const T_*)kc, (const T_*)vc, (const int*)block_tables, (const int*)seg,    \
         (const int*)pos, nh, nkv, d, page, max_blocks, q_stride, out_stride, scale, window, softcap)
     if (dtype == ILM_DTYPE_F32) {
-        if (vec) AB_LAUNCH(float, true); else AB_LAUNCH(float, false);
+        if (vec) { AB_LAUNCH(float, true); } else { AB_LAUNCH(float, false); }
     } else {
-        if (vec) AB_LAUNCH(bf16, true); else AB_LAUNCH(bf16, false);
+        if (vec) { AB_LAUNCH(bf16, true); } else { AB_LAUNCH(bf16, false); }
     }
 #undef AB_LAUNCH
+#undef AB_LAUNCH_N
     ILM_LAUNCH_CHECK("attn_basic");
     if (ws != nullptr) {
         dim3 g2(T_, nh);
-        if (dtype == ILM_DTYPE_F32)
-            attn_basic_fold_kernel<float><<<g2, 64, 0, stream>>>((float*)out, (const float*)ws, (const int*)pos, nh, d, nchunks,
-                                                                 out_stride, window);
-        else
-            attn_basic_fold_kernel<bf16><<<g2, 64, 0, stream>>>((bf16*)out, (const float*)ws, (const int*)pos, nh, d, nchunks,
-                                                                out_stride, window);
+#define AB_FOLD(T_, NA_)                                                                                              \
+    attn_basic_fold_kernel<T_, NA_><<<g2, 64, 0, stream>>>((T_*)out, (const float*)ws, (const int*)pos, nh, d, nchunks,   \
+                                                           out_stride, window)
+        if (dtype == ILM_DTYPE_F32) {
+            if (d <= 256) AB_FOLD(float, 4); else AB_FOLD(float, 16);
+        } else {
+            if (d <= 256) AB_FOLD(bf16, 4); else AB_FOLD(bf16, 16);
+        }
+#undef AB_FOLD
         ILM_LAUNCH_CHECK("attn_basic_fold");
     }
     return 0;

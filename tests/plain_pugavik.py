@@ -214,3 +214,89 @@ def tensor_shapes(cfg: dict) -> Dict[str, tuple]:
         if layer.get("mlp") is not None:
             out[p + ".mlp.up"], out[p + ".mlp.down"] = (layer["mlp"]["ff"], W), (W, layer["mlp"]["ff"])
     return out
+
+
+def greedy(cfg: dict, w: Dict[str, torch.Tensor], prompt, n: int) -> List[int]:
+    """The n tokens greedy decoding appends to `prompt` (the whole sequence is run again for every token)."""
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(torch.argmax(forward(cfg, w, toks)[-1])))
+    return toks[len(prompt):]
+
+
+def random_weights(cfg: dict, seed: int) -> Dict[str, torch.Tensor]:
+    """float32 tensors: matrices N(0, 1/in), norm weights near one, small biases, a head-mixing matrix near the identity
+    with sizeable off-diagonal entries, sinks of order one."""
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, shape in sorted(tensor_shapes(cfg).items()):
+        last = name.rsplit(".", 1)[-1]
+        if name.endswith(".talk"):
+            t = torch.eye(shape[0]) + 0.3 * torch.randn(shape, generator=g)
+        elif name.endswith(".sink"):
+            t = torch.randn(shape, generator=g)
+        elif name.endswith(".a2.b"):
+            t = 2.0 + torch.randn(shape, generator=g)                 # decays mostly near one, some fast
+        elif last == "b":
+            t = 0.1 * torch.randn(shape, generator=g)
+        elif len(shape) == 1:
+            t = 1.0 + 0.1 * torch.randn(shape, generator=g)
+        elif name in ("embed", "loop.step"):
+            t = torch.randn(shape, generator=g)
+        else:
+            t = torch.randn(shape, generator=g) / math.sqrt(shape[1])
+        out[name] = t
+    return out
+
+
+def _attention(heads, kv_heads, dim, vdim, window, rot_dims, base=10000.0, scale=None):
+    return {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "mask": {"size": window},
+            "rot": {"dims": rot_dims, "base": base}, "scale": scale if scale is not None else dim ** -0.5}
+
+
+def _latent(heads, dim, rot_dim, vdim, kv_rank, base=10000.0, scale=None):
+    return {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "rot": {"base": base, "dims": rot_dim},
+            "scale": scale if scale is not None else (dim + rot_dim) ** -0.5}
+
+
+def _gla(heads, dim, vdim, tau, decay_rank):
+    return {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau, "decay_rank": decay_rank}
+
+
+def _layer(kind, mixer, ff):
+    return {"type": kind, "mixer": mixer, "mlp": None if ff is None else {"kind": "dense", "ff": ff}}
+
+
+def config_a():
+    """No loop; a gated layer first; equal key and value sizes, as many key/value heads as heads, a part of each head turned;
+    a layer without a feed-forward."""
+    return {"architecture": "Pugavik", "vocab": 97, "width": 64, "embedding": {"scale": 1.5}, "norm": {"eps": 1e-6}, "layers": [
+        _layer("gla", _gla(2, 16, 24, 4.0, 4), 96),
+        _layer("attention", _attention(4, 4, 16, 16, 7, 8, base=100.0), None),
+        _layer("latent_attention", _latent(2, 8, 4, 12, 20), 80)]}
+
+
+def config_b():
+    """Layers 1 and 2 run three times; head sizes that are no multiples of 16 or 8; whole heads turned; one key/value head for
+    two query heads; tau 1."""
+    return {"architecture": "Pugavik", "vocab": 131, "width": 96, "embedding": {"scale": 0.7}, "norm": {"eps": 1e-5}, "layers": [
+        _layer("latent_attention", _latent(3, 16, 8, 16, 40, base=500.0), 128),
+        _layer("attention", _attention(6, 3, 12, 20, 33, 12, base=50000.0, scale=0.3), 64),
+        _layer("gla", _gla(3, 20, 8, 1.0, 6), 100),
+        _layer("attention", _attention(2, 1, 24, 8, 5, 0), 48)],
+        "loop": {"start": 1, "stop": 3, "times": 3}}
+
+
+def config_c():
+    """Sizes that take the matrix-core kernels (latent rows of 128 with the turned part, heads of 64); the first layer alone
+    runs twice; one key/value head for all heads in one layer; a window longer than most prompts."""
+    return {"architecture": "Pugavik", "vocab": 300, "width": 256, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5}, "layers": [
+        _layer("latent_attention", _latent(4, 32, 32, 64, 96), 512),
+        _layer("attention", _attention(8, 2, 64, 32, 100, 32), 384),
+        _layer("gla", _gla(4, 64, 64, 16.0, 16), 256),
+        _layer("attention", _attention(4, 1, 32, 48, 200, 16, base=1e6), None),
+        _layer("latent_attention", _latent(2, 64, 16, 32, 160), 256)],
+        "loop": {"start": 0, "stop": 1, "times": 2}}
+
+
+CONFIGS = {"A": config_a, "B": config_b, "C": config_c}
