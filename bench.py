@@ -54,6 +54,8 @@ def main() -> int:
                     help="instead of the default workload: prefill and decode throughput of the Kekevik design beside MiniCPM4 "
                          "at equal layer sizes (random weights), with the time and the roofline share of every kernel")
     ap.add_argument("--design-shapes", default="1024,4096", help="widths to compare with --designs")
+    ap.add_argument("--design", default="kekevik", choices=["kekevik", "pugavik"],
+                    help="the design that --designs puts beside MiniCPM4")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this engine has no multi-GPU path (N>1 is not run)")
@@ -92,11 +94,12 @@ def compare_designs(args) -> dict:
     from infinilm_amd.sampling import Sampler, SamplingParams
     from infinilm_amd.weights import fill_random_
     sys.path.insert(0, os.path.join(ROOT, "examples"))
-    from shapes import kekevik_shape
+    from shapes import kekevik_shape, pugavik_shape
 
     layers = 8 if args.layers == 32 else args.layers
     T, ctx, ps = args.prefill_tokens, min(args.context, 2048), args.page_size
-    out = {"metric": "prefill and decode tokens/s, Kekevik beside MiniCPM4 at equal layer sizes", "dtype": "bf16", "layers": layers,
+    design = args.design
+    out = {"metric": f"prefill and decode tokens/s, {design.capitalize()} beside MiniCPM4 at equal layer sizes", "dtype": "bf16", "layers": layers,
            "prefill_tokens": T, "context": ctx, "data": "synthetic: random weights and token ids, random-filled cache", "shapes": {}}
     sampler, greedy = Sampler(0), SamplingParams(top_k=1)
     gen = torch.Generator().manual_seed(7)
@@ -107,7 +110,7 @@ def compare_designs(args) -> dict:
                          "num_hidden_layers": layers, "hidden_size": width, "num_attention_heads": heads, "num_key_value_heads": kv,
                          "head_dim": d, "intermediate_size": 4 * width, "vocab_size": V, "max_position_embeddings": 32768,
                          "rms_norm_eps": 1e-6, "tie_word_embeddings": True},
-            "kekevik": kekevik_shape(width, heads, d, kv, layers, V, 6 * width)}
+            design: (kekevik_shape if design == "kekevik" else pugavik_shape)(width, heads, d, kv, layers, V, 6 * width)}
         rec = {}
         for name, cfg in cfgs.items():
             model = build_model(cfg, "bfloat16", "cuda:0")
@@ -181,15 +184,39 @@ def compare_designs(args) -> dict:
                     share = {}
                     state = heads * d * d * 4          # a head's state x heads (key size = value size = state entries = d here)
                     kvb = 2 * kv * d * 2               # cached bytes a token
-                    if us(rep_d, "ilm_decay_scan"):
+                    if name != "pugavik" and us(rep_d, "ilm_decay_scan"):
                         share["decay_scan decode (state read + written / HBM peak)"] = round(64 * 2 * state / us(rep_d, "ilm_decay_scan") / HBM_PEAK, 4)
                         share["decay_scan prefill (4 dk dv flops a token and head / float32 vector peak)"] = round(
                             4.0 * T * heads * d * d / us(rep_p, "ilm_decay_scan") / FLOP_PEAK["fp32"], 4)
-                    if us(rep_d, "ilm_attn_mfma"):
+                    if name != "pugavik" and us(rep_d, "ilm_attn_mfma"):
                         share["attention decode (cache read / HBM peak)"] = round(64 * ctx * kvb / us(rep_d, "ilm_attn_mfma") / HBM_PEAK, 4)
-                    if us(rep_p, "ilm_attn_tile"):
+                    if name != "pugavik" and us(rep_p, "ilm_attn_tile"):
                         share["attention prefill (4 d flops a visible key and head / bf16 matrix peak)"] = round(
                             4.0 * T * T / 2 * heads * d / us(rep_p, "ilm_attn_tile") / FLOP_PEAK["bf16"], 4)
+                    if name == "pugavik":
+                        win = 1024
+                        if us(rep_d, "ilm_attn_headmix"):
+                            seen = min(ctx, win)
+                            share["attn_headmix decode (window's cache read / HBM peak)"] = round(64 * seen * kvb / us(rep_d, "ilm_attn_headmix") / HBM_PEAK, 4)
+                            pairs = sum(min(i + 1, win) for i in range(T))
+                            share["attn_headmix prefill ((4 d + 2 heads) flops a visible key and head / float32 vector peak)"] = round(
+                                (4.0 * d + 2.0 * heads) * pairs * heads / us(rep_p, "ilm_attn_headmix") / FLOP_PEAK["fp32"], 4)
+                        gstate = heads * (d // 2) * d * 4
+                        if us(rep_d, "ilm_decay_scan"):
+                            share["decay_scan (decay per channel) decode (state read + written / HBM peak)"] = round(64 * 2 * gstate / us(rep_d, "ilm_decay_scan") / HBM_PEAK, 4)
+                            share["decay_scan (decay per channel) prefill (4 dk dv flops a token and head / float32 vector peak)"] = round(
+                                4.0 * T * heads * (d // 2) * d / us(rep_p, "ilm_decay_scan") / FLOP_PEAK["fp32"], 4)
+                        if us(rep_d, "ilm_attn_mfma"):   # (the latent layers' attention: one cached row of d entries a token, read as key and as value)
+                            share["latent attention decode (cache read / HBM peak)"] = round(64 * ctx * 2 * d * 2 / us(rep_d, "ilm_attn_mfma") / HBM_PEAK, 4)
+                        if us(rep_p, "ilm_attn_tile"):
+                            share["latent attention prefill (4 d flops a visible key and head / bf16 matrix peak)"] = round(
+                                4.0 * T * T / 2 * heads * d / us(rep_p, "ilm_attn_tile") / FLOP_PEAK["bf16"], 4)
+                        if us(rep_p, "ilm_add_layernorm"):
+                            share["add_layernorm prefill (stream read + written, two branches read, rows written / HBM peak)"] = round(
+                                T * Hs * (4 + 4 + 2 + 2 + 2) / us(rep_p, "ilm_add_layernorm") / HBM_PEAK, 4)
+                    if name == "minicpm4" and us(rep_p, "ilm_add_rmsnorm"):
+                        share["add_rmsnorm prefill (stream read + written, branch read, rows written / HBM peak)"] = round(
+                            T * Hs * (4 + 4 + 2 + 2) / us(rep_p, "ilm_add_rmsnorm") / HBM_PEAK, 4)
                     r["roofline_share"] = share
                 del runner, cache
                 torch.cuda.empty_cache()

@@ -13,11 +13,14 @@ def _factors(n: int, seed: int):
 
 
 def shape_config(name: str, layers: int = 0) -> dict:
-    """`name`: "8b", "0.5b", "2b" (MiniCPM4 family) or "kekevik-<width>" (the Kekevik design at that width, 8 layers unless
-    told otherwise); `layers` > 0 overrides the number of layers."""
+    """`name`: "8b", "0.5b", "2b" (MiniCPM4 family), "kekevik-<width>" or "pugavik-<width>" (those designs at that width,
+    8 layers unless told otherwise); `layers` > 0 overrides the number of layers."""
     if name.startswith("kekevik-"):
         width = int(name.split("-")[1])
         return kekevik_shape(width, width // 128, 128, 2, layers or 8, 32768, 6 * width)
+    if name.startswith("pugavik-"):
+        width = int(name.split("-")[1])
+        return pugavik_shape(width, width // 128, 128, 2, layers or 8, 32768, 6 * width)
     base = {"architectures": ["MiniCPMForCausalLM"], "model_type": "minicpm", "torch_dtype": "bfloat16", "rope_theta": 10000.0,
             "scale_emb": 12, "scale_depth": 1.4, "dim_model_base": 256}
     if name == "8b":
@@ -58,3 +61,24 @@ def kekevik_shape(width: int, heads: int, head_dim: int, kv_heads: int, layers: 
     kinds = [("retention", dict(lin, rot={"dims": head_dim, "base": 10000.0})), ("lightning", lin), ("parallel", par), ("parallel", par)]
     return {"architecture": "Kekevik", "vocab": vocab, "width": width, "embedding": {"scale": 12.0}, "norm": {"eps": 1e-6},
             "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]}
+
+
+def pugavik_shape(width: int, heads: int, head_dim: int, kv_heads: int, layers: int, vocab: int, ff: int, window: int = 1024,
+                  loop: dict = None) -> dict:
+    """A Pugavik configuration with the layer sizes of a transformer of this width: the three layer kinds in turn (latent
+    attention, windowed attention with mixed scores, gated linear attention), `heads` heads everywhere: query/key heads of
+    `head_dim` (the latent layers': three quarters unrotated, a quarter rotated; latent rows of three quarters of `head_dim`,
+    so that a cached row with its rotated part has `head_dim` entries), value heads of `head_dim`, gated layers with keys of
+    half of it; `ff` inner units of the feed-forward; no loop unless one is given."""
+    rot = head_dim // 4
+    latent = {"heads": heads, "dim": head_dim - rot, "rot_dim": rot, "vdim": head_dim, "kv_rank": head_dim - rot,
+              "scale": head_dim ** -0.5, "rot": {"dims": rot, "base": 10000.0}}
+    att = {"heads": heads, "kv_heads": kv_heads, "dim": head_dim, "vdim": head_dim, "scale": head_dim ** -0.5,
+           "mask": {"size": window}, "rot": {"dims": head_dim // 2, "base": 500000.0}}
+    gla = {"heads": heads, "dim": head_dim // 2, "vdim": head_dim, "tau": 16.0, "decay_rank": 16}
+    kinds = [("latent_attention", latent), ("attention", att), ("gla", gla)]
+    cfg = {"architecture": "Pugavik", "vocab": vocab, "width": width, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5},
+           "layers": [{"type": kinds[i % 3][0], "mixer": kinds[i % 3][1], "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]}
+    if loop:
+        cfg["loop"] = dict(loop)
+    return cfg

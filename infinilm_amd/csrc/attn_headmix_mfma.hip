@@ -1,0 +1,260 @@
+// Attention with scores mixed over the heads, on the matrix cores (bfloat16).
+//
+// The mixing is carried into the queries: with s_h(j) = sum_g M[h, g] scale q_g . k_kv(g),j and C key/value groups,
+//   s_h(j) = scale sum_c q'_{h,c} . k_{c,j},    q'_{h,c} = sum_{g in group c} M[h, g] q_g,
+// so head h asks with a query of C d entries against the key row [k_0,j | ... | k_{C-1},j] of all groups, and takes its
+// values from its own group.  `ilm_headmix_queries` forms q' (float sums, bfloat16 result: a query like any other
+// operand of the score product); `ilm_attn_headmix_mfma` is then a flash attention over the window with one more term
+// exp(sink_h) in the denominator.  Cost of the score product: C times that of unmixed heads, and no exchange of scores
+// between heads; for many groups the plain kernel's explicit mixing does less work.
+//
+// A workgroup = one item (a tile of up to 8 consecutive tokens of a request, or a single token) x one pass of 4 HPW
+// heads; its 4 waves take HPW heads each.  Keys go by in tiles of 32 aligned to the absolute key index; K [group][key][d]
+// and V [group][d][key] of a tile pass through LDS once for all heads of the pass.  Per head and tile:
+//   S^T [32 keys x 16 tokens] = K q'^T        (v_mfma_f32_16x16x32_bf16: A = K rows, B = q' rows; lane (r, g4) gets
+//                                              keys 4 g4 .. 4 g4 + 3 of each 16-key half for token r)
+//   running maximum, sum and weights per token (a token's keys lie in 4 lanes x 8 registers)
+//   O^T [d x 16 tokens] += V^T P^T            (A = V rows [d][key], B = the weights as they lie in the registers: the k index
+//                                              of this product is a fixed permutation of the keys, the same for A and B)
+// A token's result depends on its position and its request's cache alone: keys outside its window weigh exactly zero
+// and leave its running maximum alone, whatever other tokens share the tile.
+#include "common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 hx_bf16x8;
+typedef __attribute__((ext_vector_type(4))) float hx_f32x4;
+
+#define HX_TK 32
+#define HX_TT 8            // tokens a tile at most (the step's lists hold tiles of up to 8)
+#define HX_NEG (-1.0e30f)
+
+__device__ __forceinline__ hx_f32x4 hx_mfma(uint4 a, uint4 b, hx_f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(hx_bf16x8, a), __builtin_bit_cast(hx_bf16x8, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ uint32_t hx_pack(float lo, float hi) {
+    return (uint32_t)from_f32<bf16>(lo).bits | ((uint32_t)from_f32<bf16>(hi).bits << 16);
+}
+
+// ------------------------------------------------------------------------------------------
+// q' [T, nh, C, d] from q rows (head g at [g d, (g + 1) d)) and M [nh, nh] (null: the identity)
+// ------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+headmix_queries_kernel(bf16* __restrict__ qx, const bf16* __restrict__ q, const float* __restrict__ mix, int nh, int nkv, int d,
+                       int q_stride) {
+    extern __shared__ float qs[];
+    const int t = blockIdx.x, per = nh / nkv;
+    const bf16* row = q + (size_t)t * q_stride;
+    for (int i = threadIdx.x; i < nh * d; i += 256) qs[i] = to_f32(row[i]);
+    __syncthreads();
+    bf16* dst = qx + (size_t)t * nh * nkv * d;
+    for (int idx = threadIdx.x; idx < nh * nkv * d; idx += 256) {
+        const int e = idx % d, c = (idx / d) % nkv, h = idx / (d * nkv);
+        float a = 0.f;
+        for (int g = c * per; g < (c + 1) * per; ++g) {
+            const float m = mix != nullptr ? mix[h * nh + g] : (g == h ? 1.f : 0.f);
+            a = fmaf(m, qs[g * d + e], a);
+        }
+        dst[idx] = from_f32<bf16>(a);
+    }
+}
+
+extern "C" int ilm_headmix_queries(void* qx, const void* q, const void* mix, int T_, int nh, int nkv, int d, int q_stride,
+                                   hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && nh > 0 && nkv > 0 && nh % nkv == 0 && d > 0, "headmix_queries: bad sizes");
+    ILM_REQUIRE((size_t)nh * d * sizeof(float) <= 64 * 1024, "headmix_queries: %d heads of %d do not fit LDS", nh, d);
+    headmix_queries_kernel<<<T_, 256, (size_t)nh * d * sizeof(float), stream>>>((bf16*)qx, (const bf16*)q, (const float*)mix, nh, nkv, d,
+                                                                              q_stride);
+    ILM_LAUNCH_CHECK("headmix_queries");
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------
+template <int D32, int NC, int HPW>
+__global__ void __launch_bounds__(256)
+attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
+                         const int* __restrict__ block_tables, const int* __restrict__ seg, const int* __restrict__ pos,
+                         const int* __restrict__ tiles, int n_tiles, const int* __restrict__ singles,
+                         const float* __restrict__ sink, int nh, int page, int max_blocks, int out_stride, float scale_log2e,
+                         int window) {
+    constexpr int D = D32 * 32, KROW = D + 8, VROW = HX_TK + 8;
+    extern __shared__ __attribute__((aligned(16))) unsigned char hx_smem[];
+    bf16* Ks = reinterpret_cast<bf16*>(hx_smem);                 // [NC][32][KROW]
+    bf16* Vs = Ks + NC * HX_TK * KROW;                           // [NC][D][VROW]
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g4 = lane >> 4, wave = tid >> 6;
+    int t0, ntok;
+    if ((int)blockIdx.x < n_tiles) {
+        t0 = tiles[2 * blockIdx.x];
+        ntok = tiles[2 * blockIdx.x + 1];
+    } else {
+        const int i = blockIdx.x - n_tiles;
+        t0 = singles != nullptr ? singles[i] : i;
+        ntok = t0 >= 0 ? 1 : 0;
+    }
+    if (ntok <= 0) return;                                       // an entry that fills up a recorded step's lists
+    const int p_first = pos[t0], p_last = p_first + ntok - 1;
+    const int lo_first = (window > 0 && p_first - window + 1 > 0) ? p_first - window + 1 : 0;
+    const int* bt = block_tables + (size_t)seg[t0] * max_blocks;
+    const int per = nh / NC;
+    // this lane's token (column r of the products)
+    const bool tok_ok = r < ntok;
+    const int tok = t0 + (tok_ok ? r : 0);
+    const int p_tok = p_first + (tok_ok ? r : 0);
+    const int lo_tok = (window > 0 && p_tok - window + 1 > 0) ? p_tok - window + 1 : 0;
+    // this wave's heads and their queries
+    int head[HPW];
+    bool head_ok[HPW];
+    uint4 qf[HPW][NC][D32];
+    hx_f32x4 O[HPW][2 * D32];
+    float m_run[HPW], l_run[HPW];
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+        const int h = (blockIdx.y * 4 + wave) * HPW + i;
+        head_ok[i] = h < nh;
+        head[i] = head_ok[i] ? h : nh - 1;
+        const bf16* qrow = qx + ((size_t)tok * nh + head[i]) * NC * D;
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+#pragma unroll
+            for (int ks = 0; ks < D32; ++ks) qf[i][c][ks] = *reinterpret_cast<const uint4*>(qrow + c * D + ks * 32 + g4 * 8);
+#pragma unroll
+        for (int b = 0; b < 2 * D32; ++b) O[i][b] = hx_f32x4{0.f, 0.f, 0.f, 0.f};
+        m_run[i] = HX_NEG;
+        l_run[i] = 0.f;
+    }
+    constexpr int KPIECES = NC * HX_TK * (D / 8), VPIECES = NC * D * (HX_TK / 8);
+    const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
+    for (int kb = lo_first & ~(HX_TK - 1); kb <= p_last; kb += HX_TK) {
+        const int pg = bt[kb / page];                            // (a tile lies on one page: the page size is a multiple of 32)
+        const int off = kb % page;
+        __syncthreads();                                         // the tile before this one has been read by every wave
+        for (int pc = tid; pc < KPIECES; pc += 256) {
+            const int c = pc / (HX_TK * (D / 8)), rest = pc % (HX_TK * (D / 8)), key = rest / (D / 8), piece = rest % (D / 8);
+            uint4 v = zero4;
+            if (pg >= 0) v = *reinterpret_cast<const uint4*>(kc + (((size_t)pg * NC + c) * page + off + key) * D + piece * 8);
+            *reinterpret_cast<uint4*>(Ks + (c * HX_TK + key) * KROW + piece * 8) = v;
+        }
+        for (int pc = tid; pc < VPIECES; pc += 256) {
+            const int c = pc / (D * (HX_TK / 8)), rest = pc % (D * (HX_TK / 8)), row = rest / (HX_TK / 8), piece = rest % (HX_TK / 8);
+            uint4 v = zero4;
+            if (pg >= 0) v = *reinterpret_cast<const uint4*>(vc + (((size_t)pg * NC + c) * D + row) * page + off + piece * 8);
+            *reinterpret_cast<uint4*>(Vs + (c * D + row) * VROW + piece * 8) = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < HPW; ++i) {
+            if (!head_ok[i]) continue;                           // (uniform over the wave)
+            hx_f32x4 S[2];
+#pragma unroll
+            for (int s = 0; s < 2; ++s) {
+                S[s] = hx_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < NC; ++c)
+#pragma unroll
+                    for (int ks = 0; ks < D32; ++ks) {
+                        const uint4 a = *reinterpret_cast<const uint4*>(Ks + (c * HX_TK + s * 16 + r) * KROW + ks * 32 + g4 * 8);
+                        S[s] = hx_mfma(a, qf[i][c][ks], S[s]);
+                    }
+            }
+            // this lane: token r, keys kb + 16 s + 4 g4 + j
+            float sc[8];
+            float mx = HX_NEG;
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int key = kb + s * 16 + g4 * 4 + j;
+                    const bool seen = tok_ok && key >= lo_tok && key <= p_tok;
+                    sc[s * 4 + j] = seen ? S[s][j] * scale_log2e : HX_NEG;
+                    mx = fmaxf(mx, sc[s * 4 + j]);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            const float m_new = fmaxf(m_run[i], mx);
+            const float corr = __builtin_amdgcn_exp2f(m_run[i] - m_new);
+            float pw[8], sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                pw[j] = sc[j] > 0.5f * HX_NEG ? __builtin_amdgcn_exp2f(sc[j] - m_new) : 0.f;
+                sum += pw[j];
+            }
+            l_run[i] = l_run[i] * corr + sum;                    // (this lane's share; the four lanes of a token are summed at the end)
+            m_run[i] = m_new;
+            const uint4 pb = make_uint4(hx_pack(pw[0], pw[1]), hx_pack(pw[2], pw[3]), hx_pack(pw[4], pw[5]), hx_pack(pw[6], pw[7]));
+            const int c_h = head[i] / per;
+#pragma unroll
+            for (int b = 0; b < 2 * D32; ++b) {
+                const bf16* vrow = Vs + (c_h * D + b * 16 + r) * VROW;
+                const uint2 v0 = *reinterpret_cast<const uint2*>(vrow + g4 * 4);          // keys 4 g4 .. + 3
+                const uint2 v1 = *reinterpret_cast<const uint2*>(vrow + 16 + g4 * 4);     // keys 16 + 4 g4 .. + 3
+                hx_f32x4 o = O[i][b];
+                o[0] *= corr; o[1] *= corr; o[2] *= corr; o[3] *= corr;
+                O[i][b] = hx_mfma(make_uint4(v0.x, v0.y, v1.x, v1.y), pb, o);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < HPW; ++i) {
+        if (!head_ok[i]) continue;
+        float l = l_run[i];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        if (sink != nullptr) l += __builtin_amdgcn_exp2f(sink[head[i]] * 1.4426950408889634f - m_run[i]);
+        const float inv = 1.0f / l;
+        if (tok_ok) {
+            bf16* orow = out + (size_t)tok * out_stride + (size_t)head[i] * D;
+#pragma unroll
+            for (int b = 0; b < 2 * D32; ++b) {
+                const hx_f32x4 o = O[i][b];
+                *reinterpret_cast<uint2*>(orow + b * 16 + g4 * 4) = make_uint2(hx_pack(o[0] * inv, o[1] * inv), hx_pack(o[2] * inv, o[3] * inv));
+            }
+        }
+    }
+}
+
+extern "C" int ilm_attn_headmix_mfma_ok(int nh, int nkv, int d, int page) {
+    return nh > 0 && nkv > 0 && nh % nkv == 0 && (nkv == 1 || nkv == 2 || nkv == 4) && d % 32 == 0 && d >= 32 && d <= 128 &&
+           page % HX_TK == 0;
+}
+
+// qx [T, nh, nkv, d] from ilm_headmix_queries; tiles [n_tiles, 2] = (first row, count <= 8) and n_singles single rows
+// (`singles` null: rows 0 .. n_singles - 1; an entry -1 or a count 0 names nothing)
+extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, const void* vc, const void* block_tables,
+                                     const void* seg, const void* pos, const void* tiles, int n_tiles, const void* singles,
+                                     int n_singles, const void* sink, int nh, int nkv, int d, int page, int max_blocks,
+                                     int out_stride, float scale, int window, hipStream_t stream) {
+    ILM_REQUIRE(n_tiles >= 0 && n_singles >= 0 && n_tiles + n_singles > 0 && max_blocks > 0, "attn_headmix_mfma: bad sizes");
+    ILM_REQUIRE(ilm_attn_headmix_mfma_ok(nh, nkv, d, page), "attn_headmix_mfma: %d heads in %d groups of %d, pages of %d", nh, nkv, d, page);
+    ILM_REQUIRE(out_stride % 4 == 0 && ((uintptr_t)out & 7) == 0 && ((uintptr_t)qx & 15) == 0 && ((uintptr_t)kc & 15) == 0 &&
+                ((uintptr_t)vc & 15) == 0, "attn_headmix_mfma: rows must be 16-byte / 8-byte aligned");
+    const float scale_log2e = scale * 1.4426950408889634f;
+#define HX_LAUNCH(D32_, NC_, HPW_)                                                                                         \
+    {                                                                                                                      \
+        auto kern = attn_headmix_mfma_kernel<D32_, NC_, HPW_>;                                                             \
+        const int shm = NC_ * HX_TK * (D32_ * 32 + 8) * 2 + NC_ * D32_ * 32 * (HX_TK + 8) * 2;                             \
+        if (shm > 48 * 1024) {                                                                                             \
+            hipError_t e_ = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm);       \
+            ILM_REQUIRE(e_ == hipSuccess, "attn_headmix_mfma: %d bytes of LDS refused: %s", shm, hipGetErrorString(e_));   \
+        }                                                                                                                  \
+        dim3 grid(n_tiles + n_singles, (nh + 4 * HPW_ - 1) / (4 * HPW_));                                                  \
+        kern<<<grid, 256, shm, stream>>>((bf16*)out, (const bf16*)qx, (const bf16*)kc, (const bf16*)vc,                    \
+                                         (const int*)block_tables, (const int*)seg, (const int*)pos, (const int*)tiles,    \
+                                         n_tiles, (const int*)singles, (const float*)sink, nh, page, max_blocks,           \
+                                         out_stride, scale_log2e, window);                                                 \
+    }
+#define HX_BY_NC(D32_)                                                      \
+    switch (nkv) {                                                          \
+        case 1: HX_LAUNCH(D32_, 1, 4) break;                                \
+        case 2: if (D32_ <= 2) HX_LAUNCH(D32_, 2, 4) else HX_LAUNCH(D32_, 2, 2) break; \
+        default: if (D32_ <= 2) HX_LAUNCH(D32_, 4, 2) else HX_LAUNCH(D32_, 4, 1) break; \
+    }
+    switch (d / 32) {
+        case 1: HX_BY_NC(1) break;
+        case 2: HX_BY_NC(2) break;
+        case 3: HX_BY_NC(3) break;
+        default: HX_BY_NC(4) break;
+    }
+#undef HX_BY_NC
+#undef HX_LAUNCH
+    ILM_LAUNCH_CHECK("attn_headmix_mfma");
+    return 0;
+}

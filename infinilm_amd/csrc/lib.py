@@ -53,10 +53,12 @@ _SIGNATURES = {
     "ilm_unary": [_P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "ilm_lin_prep": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "ilm_decay_scan": [_P, _I, _P, _P, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P],
-    "ilm_sigmoid_root": [_P, _P, _I, _I, _I, _I, _F, _I, _P],
+    "ilm_sigmoid_root": [_P, _P, _P, _I, _I, _I, _I, _F, _I, _I, _P],
     "ilm_add_layernorm": [_P, _P, _P, _P, _I, _I, _F, _I, _I, _I] + [_P, _I, _I, _L, _L, _F] * 4 + [_P],
     "ilm_qkv_norm_rope_kvwrite": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
     "ilm_attn_headmix": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "ilm_headmix_queries": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
+    "ilm_attn_headmix_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "ilm_latent_prep": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
     "ilm_head_gemm": [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _I, _I, _P],
     "ilm_group_norm_gate": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _I, _I, _L, _P],
@@ -100,6 +102,8 @@ def load(verbose: bool = True) -> ctypes.CDLL:
                                "(python -c 'import __graft_entry__ as g; g.build()')")
         fn.argtypes = args
         fn.restype = c_int
+    lib.ilm_attn_headmix_mfma_ok.restype = c_int
+    lib.ilm_attn_headmix_mfma_ok.argtypes = [c_int, c_int, c_int, c_int]
     lib.ilm_attn_static_init.restype = c_int
     lib.ilm_attn_static_init.argtypes = []
     lib.ilm_attn_static_scratch_floats.restype = c_long

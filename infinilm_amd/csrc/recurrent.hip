@@ -109,32 +109,38 @@ extern "C" int ilm_unary(void* out, const void* in, int T_, int n, int out_strid
 }
 
 // ------------------------------------------------------------------------------------------
-// Decays of a gated recurrence from their raw rows: out[t, j] = sigmoid(z[t, j])^inv_tau = exp(inv_tau * log sigmoid(z)),
-// the logarithm in its stable form (-log1p(exp(-z)) for z >= 0, z - log1p(exp(z)) below); float results.
+// Decays of a gated recurrence from their raw rows: out[t, j] = sigmoid(z[t, j] + b[j])^inv_tau = exp(inv_tau * log
+// sigmoid(.)), the logarithm in its stable form (-log1p(exp(-x)) for x >= 0, x - log1p(exp(x)) below); float results.
 // ------------------------------------------------------------------------------------------
-template <typename T>
+template <typename T, typename TB>
 __global__ void __launch_bounds__(256)
-sigmoid_root_kernel(float* __restrict__ out, const T* __restrict__ z, int n, int out_stride, int in_stride, float inv_tau) {
+sigmoid_root_kernel(float* __restrict__ out, const T* __restrict__ z, const TB* __restrict__ bias, int n, int out_stride,
+                    int in_stride, float inv_tau) {
     const int t = blockIdx.y, j = blockIdx.x * 256 + threadIdx.x;
     if (j >= n) return;
-    const float x = to_f32(z[(size_t)t * in_stride + j]);
+    const float x = to_f32(z[(size_t)t * in_stride + j]) + (bias != nullptr ? to_f32(bias[j]) : 0.f);
     const float ls = x >= 0.f ? -log1pf(expf(-x)) : x - log1pf(expf(x));
     out[(size_t)t * out_stride + j] = expf(inv_tau * ls);
 }
 
-extern "C" int ilm_sigmoid_root(void* out, const void* z, int T_, int n, int out_stride, int in_stride, float inv_tau, int z_dt,
-                                hipStream_t stream) {
-    ILM_REQUIRE(T_ > 0 && n > 0 && T_ <= 65535 * 32, "sigmoid_root: bad sizes");
+extern "C" int ilm_sigmoid_root(void* out, const void* z, const void* bias, int T_, int n, int out_stride, int in_stride,
+                                float inv_tau, int z_dt, int b_dt, hipStream_t stream) {
+    ILM_REQUIRE(T_ > 0 && n > 0, "sigmoid_root: bad sizes");
     ILM_REQUIRE(z_dt == ILM_DTYPE_F32 || z_dt == ILM_DTYPE_BF16, "sigmoid_root: unknown dtype %d", z_dt);
+    ILM_REQUIRE(bias == nullptr || b_dt == ILM_DTYPE_F32 || b_dt == ILM_DTYPE_BF16, "sigmoid_root: unknown bias dtype %d", b_dt);
     for (int t0 = 0; t0 < T_; t0 += 65535) {
         const int rows = T_ - t0 < 65535 ? T_ - t0 : 65535;
         dim3 grid((n + 255) / 256, rows);
-        if (z_dt == ILM_DTYPE_F32)
-            sigmoid_root_kernel<float><<<grid, 256, 0, stream>>>((float*)out + (size_t)t0 * out_stride,
-                                                                 (const float*)z + (size_t)t0 * in_stride, n, out_stride, in_stride, inv_tau);
-        else
-            sigmoid_root_kernel<bf16><<<grid, 256, 0, stream>>>((float*)out + (size_t)t0 * out_stride,
-                                                                (const bf16*)z + (size_t)t0 * in_stride, n, out_stride, in_stride, inv_tau);
+        float* o = (float*)out + (size_t)t0 * out_stride;
+#define SR_LAUNCH(T__, TB__)                                                                                          \
+    sigmoid_root_kernel<T__, TB__><<<grid, 256, 0, stream>>>(o, (const T__*)z + (size_t)t0 * in_stride, (const TB__*)bias, n, \
+                                                             out_stride, in_stride, inv_tau)
+        if (z_dt == ILM_DTYPE_F32) {
+            if (b_dt == ILM_DTYPE_BF16) SR_LAUNCH(float, bf16); else SR_LAUNCH(float, float);
+        } else {
+            if (b_dt == ILM_DTYPE_BF16) SR_LAUNCH(bf16, bf16); else SR_LAUNCH(bf16, float);
+        }
+#undef SR_LAUNCH
     }
     ILM_LAUNCH_CHECK("sigmoid_root");
     return 0;

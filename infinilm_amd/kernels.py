@@ -374,6 +374,11 @@ def gemm(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, 
         _run("ilm_gemm_skinny", out.data_ptr(), a.data_ptr(), w.data_ptr(), _ptr(bias), M, N, K, a.stride(0),
              w.stride(0), out.stride(0), float(alpha), _DT[out_dtype], SKINNY_VARIANT, _stream())
         return out
+    if M > 16 and fast and bias is not None and alpha == 1.0 and out_dtype == BF16 and USE_LIBRARY_GEMM:
+        # many rows with a bias: the vendor library's product with the bias row as its addend
+        with _timed("library_gemm"):
+            torch.addmm(bias, a, w.t(), out=out)
+        return out
     if M > 16 and library_ok:
         # large products go to the vendor library, as the reference's linear layers do
         # (csrc/layers/quantization/none_quantization.cpp:26-46 calls its library's linear)
@@ -1123,14 +1128,17 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, dk
     return o
 
 
-def sigmoid_root(z: torch.Tensor, tau: float) -> torch.Tensor:
-    """float32 sigmoid(z)^(1/tau), element by element (the decays of a gated recurrence from their raw rows); z [T, n]
-    with dense rows."""
-    _dev(z)
+def sigmoid_root(z: torch.Tensor, tau: float, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 sigmoid(z + bias)^(1/tau), element by element (the decays of a gated recurrence from their raw rows); z [T, n]
+    with dense rows, `bias` [n] or None."""
+    _dev(z, bias)
     _rows(z, "z")
     T, n = z.shape
+    if bias is not None and (bias.shape != (n,) or not bias.is_contiguous()):
+        raise KernelError(f"bias must be contiguous [{n}]")
     out = torch.empty((T, n), dtype=F32, device=z.device)
-    _run("ilm_sigmoid_root", out.data_ptr(), z.data_ptr(), T, n, out.stride(0), z.stride(0), 1.0 / float(tau), _dt(z), _stream())
+    _run("ilm_sigmoid_root", out.data_ptr(), z.data_ptr(), _ptr(bias), T, n, out.stride(0), z.stride(0), 1.0 / float(tau), _dt(z),
+         _dt(bias) if bias is not None else 0, _stream())
     return out
 
 
@@ -1312,6 +1320,9 @@ def add_layernorm(residual: torch.Tensor, addends, weight: Optional[torch.Tensor
 
 
 # ---- attention with scores mixed over the heads ----------------------------------------------------
+USE_HEADMIX_MFMA = os.environ.get("INFINILM_AMD_HEADMIX_MFMA", "1") == "1"   # 0: always the plain kernel
+
+
 def qkv_norm_rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, freq: Optional[torch.Tensor], q_weight: Optional[torch.Tensor],
                           k_weight: Optional[torch.Tensor], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
                           slots: Optional[torch.Tensor], nh: int, nkv: int, d: int, dn: int, dv: int, rd: int, v_norm: bool,
@@ -1345,11 +1356,15 @@ def qkv_norm_rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, freq: Opti
 
 def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                       seg_of_token: torch.Tensor, positions: torch.Tensor, nh: int, nkv: int, d: int, dv: int, scale: float,
-                      window: int = 0, mix: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      window: int = 0, mix: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
+                      tiles: Optional[torch.Tensor] = None, single_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of every token over its request's cached keys (its last `window` positions, or all) where the scaled
     scores of the heads are mixed before the softmax, s_h = sum_g mix[h, g] raw_g (`mix` float32 [nh, nh] or None),
     and every head's denominator holds one more term exp(sink[h]) (`sink` float32 [nh] or None).  q, caches, block
-    tables as for `paged_attention`; `dv`: the entries of a value head that count.  Returns [T, nh*d]."""
+    tables as for `paged_attention`; `dv`: the entries of a value head that count.  `tiles` [n, 2] = (first row, count <=
+    ATT_TILE_TOKENS) lists runs of consecutive tokens of one request and `single_rows` the remaining rows (without them
+    every token is served on its own); the matrix-core kernel (bfloat16, heads of 32 to 128 in steps of 32, 1, 2 or 4
+    key/value groups, pages of a multiple of 32) works by them, the plain kernel token by token.  Returns [T, nh*d]."""
     _dev(q, k_cache, v_cache, block_tables, seg_of_token, positions, mix, sink)
     _i32(block_tables, "block_tables")
     _i32(seg_of_token, "seg_of_token")
@@ -1367,6 +1382,22 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     if sink is not None and (sink.dtype != F32 or tuple(sink.shape) != (nh,) or not sink.is_contiguous()):
         raise KernelError(f"the denominators' extra terms must be contiguous float32 [{nh}]")
     out = torch.empty((T, nh * d), dtype=q.dtype, device=q.device)
+    if (q.dtype == BF16 and not FORCE_BASIC and USE_HEADMIX_MFMA and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0
+            and _lib().ilm_attn_headmix_mfma_ok(nh, nkv, d, page)):
+        # the mixing carried into the queries, then a flash attention on the matrix cores
+        qx = torch.empty((T, nh, nkv, d), dtype=BF16, device=q.device)
+        _run("ilm_headmix_queries", qx.data_ptr(), q.data_ptr(), _ptr(mix), T, nh, nkv, d, q.stride(0), _stream())
+        n_tiles, n_single, rows = 0, T, None
+        if tiles is not None and tiles.numel() > 0:
+            _i32(tiles, "tiles")
+            n_tiles, n_single = tiles.numel() // 2, 0
+            if single_rows is not None and single_rows.numel() > 0:
+                _i32(single_rows, "single_rows")
+                rows, n_single = single_rows, single_rows.numel()
+        _run("ilm_attn_headmix_mfma", out.data_ptr(), qx.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
+             seg_of_token.data_ptr(), positions.data_ptr(), _ptr(tiles) if n_tiles else None, n_tiles, _ptr(rows), n_single,
+             _ptr(sink), nh, nkv, d, page, block_tables.shape[1], out.stride(0), float(scale), int(window), _stream())
+        return out
     _run("ilm_attn_headmix", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
          seg_of_token.data_ptr(), positions.data_ptr(), None, T, _ptr(mix), _ptr(sink), nh, nkv, d, int(dv), page,
          block_tables.shape[1], q.stride(0), out.stride(0), float(scale), int(window), _dt(q), _stream())

@@ -152,8 +152,9 @@ class GatedLinearAttention(Mixer):
         H, dk, dv = self.H, self.dk, self.dv
         rows = self.proj.forward(x)                                    # [T, q | k | v | g | low]
         g0 = 2 * H * dk + H * dv
-        z = self.a2.forward(rows[:, g0 + H * dv:], out_dtype=torch.float32)          # [T, heads * dk]
-        alpha = kernels.sigmoid_root(z, self.tau)
+        # the low-rank pair's second product without its bias (float32 result), the bias inside the decays' kernel
+        z = kernels.gemm(rows[:, g0 + H * dv:], self.a2.weight, None, 1.0, torch.float32)          # [T, heads * dk]
+        alpha = kernels.sigmoid_root(z, self.tau, bias=self.a2.bias)
         f = kernels.linear_attention_inputs(rows, None, None, H, dk, dv, 0, "none", float(dk) ** -0.5)
         o = kernels.decay_scan(f[:, :H * dk], f[:, H * dk:2 * H * dk], f[:, 2 * H * dk:], H, dk, dv, H, view.pool,
                                view.state_in, view.state_out, batch.seg_offsets, view.state_in.numel(), decay_c=alpha)

@@ -106,6 +106,61 @@ def test_sigmoid_root_is_stable_at_both_ends():
         _close(got, want, 1e-6, f"tau {tau}")
     got = kernels.sigmoid_root(z.to(torch.bfloat16).to(DEV), 2.0).cpu().double()
     _close(got, torch.exp(-torch.nn.functional.softplus(-z.to(torch.bfloat16).double()) / 2.0), 1e-6, "bfloat16 rows")
+    bias = torch.linspace(-2.0, 2.0, 9)
+    got = kernels.sigmoid_root(z.to(DEV), 4.0, bias=bias.to(DEV)).cpu().double()
+    _close(got, torch.exp(-torch.nn.functional.softplus(-(z + bias).double()) / 4.0), 1e-6, "with a bias")
+
+
+@pytest.mark.parametrize("window", [0, 5, 40, 1000])
+@pytest.mark.parametrize("nh,nkv,d,dv", [(8, 2, 64, 32), (4, 1, 128, 128), (8, 4, 32, 20), (32, 2, 128, 96), (6, 2, 96, 96), (20, 4, 128, 128)])
+def test_matrix_core_headmix_attention_equals_the_plain_kernel(nh, nkv, d, dv, window):
+    """A step with a portion of 19 tokens after 70 cached ones (tiles of 8, 8 and 3 tokens), a decoded token at position 130
+    of another request (pages the window has passed are gone) and a first token of a third: the matrix-core kernel against
+    the plain one on the same cache, and the plain one against the formula."""
+    from infinilm_amd import kernels
+    g = torch.Generator().manual_seed(nh * 7 + d + window)
+    page, pages = 32, 12
+    bf = torch.bfloat16
+    kc = torch.randn(pages + 1, nkv, page, d, generator=g).to(bf)
+    vc = torch.randn(pages + 1, nkv, d, page, generator=g).to(bf)
+    vc[:, :, dv:] = 0
+    lens = [89, 131, 1]                                    # keys of each request after this step
+    tables = [[3, 7, 1, -1, -1], [9, 2, 10, 4, 6], [5, -1, -1, -1, -1]]
+    if 0 < window <= 40:                                   # pages the decoded token's window has passed are given back
+        tables[1][:(131 - window) // page] = [-1] * ((131 - window) // page)
+    rows_pos = [(0, 70 + i) for i in range(19)] + [(1, 130), (2, 0)]
+    T = len(rows_pos)
+    q = torch.randn(T, nh * d, generator=g).to(bf)
+    mix = (torch.eye(nh) + 0.3 * torch.randn(nh, nh, generator=g)).float()
+    sink = torch.randn(nh, generator=g).float()
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    args = (q.to(DEV), kc.to(DEV), vc.to(DEV), i32(tables), i32([r for r, _ in rows_pos]), i32([p for _, p in rows_pos]), nh, nkv, d, dv,
+            d ** -0.5, window)
+    tiles, singles = i32([[0, 8], [8, 8], [16, 3], [0, 0]]), i32([19, -1, 20])
+    fast = kernels.headmix_attention(*args, mix=mix.to(DEV), sink=sink.to(DEV), tiles=tiles, single_rows=singles).cpu()
+    each = kernels.headmix_attention(*args, mix=mix.to(DEV), sink=sink.to(DEV)).cpu()
+    old = kernels.USE_HEADMIX_MFMA
+    kernels.USE_HEADMIX_MFMA = False
+    try:
+        plain = kernels.headmix_attention(*args, mix=mix.to(DEV), sink=sink.to(DEV)).cpu()
+    finally:
+        kernels.USE_HEADMIX_MFMA = old
+    # the formula, request by request
+    want = torch.zeros(T, nh, d, dtype=torch.float64)
+    per = nh // nkv
+    for t, (r, p) in enumerate(rows_pos):
+        lo = max(0, p - window + 1) if window > 0 else 0
+        keys = torch.stack([kc[tables[r][j // page], :, j % page, :] for j in range(lo, p + 1)]).double()      # [n, nkv, d]
+        vals = torch.stack([vc[tables[r][j // page], :, :, j % page] for j in range(lo, p + 1)]).double()
+        raw = torch.stack([keys[:, h // per] @ q[t].double().view(nh, d)[h] for h in range(nh)]) * d ** -0.5       # [nh, n]
+        s = mix.double() @ raw
+        top = torch.maximum(s.max(-1).values, sink.double())
+        e = torch.exp(s - top[:, None])
+        prob = e / (e.sum(-1) + torch.exp(sink.double() - top))[:, None]
+        want[t] = torch.stack([prob[h] @ vals[:, h // per] for h in range(nh)])
+    _close(plain.view(T, nh, d), want, 1e-2, "the plain kernel against the formula")
+    _close(fast.view(T, nh, d), want, 2e-2, "the matrix-core kernel, by tiles")
+    _close(each.view(T, nh, d), want, 2e-2, "the matrix-core kernel, token by token")
 
 
 @pytest.mark.parametrize("heads,dk,dv", [(2, 16, 24), (3, 5, 3), (2, 128, 64), (1, 200, 40), (4, 64, 8)])
