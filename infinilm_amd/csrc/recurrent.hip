@@ -401,14 +401,17 @@ decay_scan_kernel(float* __restrict__ o, int o_stride, const float* __restrict__
 // computed (one barrier a tile), instead of every thread loading its own entries token by token: a wave then waits for
 // memory once a tile, not once a token.  Thread (kp, column group) owns the SC_NK consecutive state entries
 // kp * SC_NK ... of its VC columns.  LDS: 2 buffers x TB x (2 dkp + columns + 2) floats, dkp = KP * SC_NK.
-template <int MODE, int VC>
+// CH: a decay per token, head and key channel (decay_c, rows dc_stride apart): the tile holds the decays beside q and k,
+// and a piece's product of decays is a vector of dk numbers a head (ws_decay [slots][heads][dk]).
+template <int MODE, int VC, bool CH = false>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3)))   // (three blocks a compute unit: 168 registers)
 decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __restrict__ q, const float* __restrict__ k,
                         int qk_stride, int q_div, const float* __restrict__ v, int v_stride,
                         const float* __restrict__ decay_h, const float* __restrict__ decay_t,
                         const float* __restrict__ kscale_t, const float* __restrict__ skip_h,
                         const int* __restrict__ seg_offsets, int heads, int dk, int dv, int KP, int R, int piece, int TB,
-                        float* __restrict__ ws_state, float* __restrict__ ws_decay) {
+                        float* __restrict__ ws_state, float* __restrict__ ws_decay, const float* __restrict__ decay_c = nullptr,
+                        int dc_stride = 0) {
     extern __shared__ float lds[];
     const int h = blockIdx.y, slot = blockIdx.z;
     int p;
@@ -420,7 +423,7 @@ decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __rest
     const int vb = blockIdx.x * cols;                                 // first column of the block
     const size_t hs = (size_t)dk * dv;
     float* st = ws_state + ((size_t)slot * heads + h) * hs;
-    const int per = TB * (2 * dkp + cols + 2);                        // floats of one buffer: q | k | v | a | b
+    const int per = TB * ((CH ? 3 : 2) * dkp + cols + 2);             // floats of one buffer: q | k | v | a | b (| decays per channel)
     float S[VC][SC_NK];
 #pragma unroll
     for (int c = 0; c < VC; ++c)
@@ -432,7 +435,7 @@ decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __rest
     const int qoff = (h / q_div) * dk;
     const float a_h = decay_h != nullptr ? decay_h[h] : 1.0f;
     const float skip = skip_h != nullptr ? skip_h[h] : 0.f;
-    float rq[8], rk[8], rv[8], ra = 1.f, rb = 1.f;     // a tile on its way: TB * dkp <= 2048 and TB * cols <= 2048
+    float rq[8], rk[8], rv[8], rc[CH ? 8 : 1], ra = 1.f, rb = 1.f;     // a tile on its way: TB * dkp <= 2048 and TB * cols <= 2048
 #define SCT_FETCH(T0_)                                                                                       \
     {                                                                                                        \
         _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                                      \
@@ -441,6 +444,7 @@ decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __rest
             const size_t at = (size_t)((T0_) + tt) * qk_stride + qoff + ki;                                  \
             rq[i] = (MODE == SC_FROM && ok) ? q[at] : 0.f;                                                   \
             rk[i] = ok ? k[at] : 0.f;                                                                        \
+            if (CH) rc[CH ? i : 0] = ok ? decay_c[(size_t)((T0_) + tt) * dc_stride + (size_t)h * dk + ki] : 1.f; \
         }                                                                                                    \
         _Pragma("unroll") for (int i = 0; i < 8; ++i) {                                                      \
             const int idx = threadIdx.x + i * 256, tt = idx / cols, c = idx % cols;                          \
@@ -460,6 +464,7 @@ decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __rest
             if (idx < TB * dkp) {                                                                            \
                 b_[idx] = rq[i];                                                                             \
                 b_[TB * dkp + idx] = rk[i];                                                                  \
+                if (CH) b_[TB * (2 * dkp + cols + 2) + idx] = rc[CH ? i : 0];                                \
             }                                                                                                \
             if (idx < TB * cols) b_[2 * TB * dkp + idx] = rv[i];                                             \
         }                                                                                                    \
@@ -471,7 +476,9 @@ decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __rest
     SCT_FETCH(t0)
     SCT_STORE(0)
     __syncthreads();
-    float aprod = 1.0f;
+    float aprod = 1.0f, aprodc[CH ? SC_NK : 1];
+#pragma unroll
+    for (int i = 0; i < (CH ? SC_NK : 1); ++i) aprodc[i] = 1.0f;
     int buf = 0;
     for (int tb = t0; tb < t1; tb += TB, buf ^= 1) {
         const bool more = tb + TB < t1;
@@ -480,7 +487,7 @@ decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __rest
         const int n = min(TB, t1 - tb);
 #pragma unroll 2
         for (int tt = 0; tt < n; ++tt) {
-            float qc[SC_NK], kc[SC_NK], vcur[VC];
+            float qc[SC_NK], kc[SC_NK], vcur[VC], ac[SC_NK];
             const float a = b_[TB * (2 * dkp + cols) + tt], bsc = b_[TB * (2 * dkp + cols + 1) + tt];
 #pragma unroll
             for (int i4 = 0; i4 < SC_NK; i4 += 4) {
@@ -490,6 +497,12 @@ decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __rest
                 }
                 const float4 u4 = *reinterpret_cast<const float4*>(b_ + TB * dkp + tt * dkp + kp * SC_NK + i4);
                 kc[i4] = u4.x * bsc; kc[i4 + 1] = u4.y * bsc; kc[i4 + 2] = u4.z * bsc; kc[i4 + 3] = u4.w * bsc;
+                if (CH) {
+                    const float4 w4 = *reinterpret_cast<const float4*>(b_ + TB * (2 * dkp + cols + 2) + tt * dkp + kp * SC_NK + i4);
+                    ac[i4] = w4.x; ac[i4 + 1] = w4.y; ac[i4 + 2] = w4.z; ac[i4 + 3] = w4.w;
+                } else {
+                    ac[i4] = ac[i4 + 1] = ac[i4 + 2] = ac[i4 + 3] = a;
+                }
             }
 #pragma unroll
             for (int c = 0; c < VC; ++c) vcur[c] = b_[2 * TB * dkp + tt * cols + cl + c];
@@ -499,12 +512,16 @@ decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __rest
                 acc[c] = 0.f;
 #pragma unroll
                 for (int i = 0; i < SC_NK; ++i) {
-                    S[c][i] = fmaf(a, S[c][i], kc[i] * vcur[c]);
+                    S[c][i] = fmaf(ac[i], S[c][i], kc[i] * vcur[c]);
                     if (MODE == SC_FROM) acc[c] = fmaf(S[c][i], qc[i], acc[c]);
                 }
             }
             if (MODE == SC_LOCAL) {
                 aprod *= a;
+                if (CH) {
+#pragma unroll
+                    for (int i = 0; i < SC_NK; ++i) aprodc[CH ? i : 0] *= ac[i];
+                }
             } else {
                 if (VC == 4 && KP >= 4) {
                     const float (&a4)[4] = reinterpret_cast<const float (&)[4]>(acc);
@@ -536,14 +553,23 @@ decay_scan_tiled_kernel(float* __restrict__ o, int o_stride, const float* __rest
             const int ki = kp * SC_NK + i, vc = vb + cl + c;
             if (vc < dv && ki < dk) st[(size_t)vc * dk + ki] = S[c][i];
         }
-    if (blockIdx.x == 0 && threadIdx.x == 0) ws_decay[(size_t)slot * heads + h] = aprod;
+    if (CH) {
+        if (blockIdx.x == 0 && threadIdx.x < KP)
+#pragma unroll
+            for (int i = 0; i < SC_NK; ++i) {
+                const int ki = kp * SC_NK + i;
+                if (ki < dk) ws_decay[((size_t)slot * heads + h) * dk + ki] = aprodc[CH ? i : 0];
+            }
+    } else if (blockIdx.x == 0 && threadIdx.x == 0) {
+        ws_decay[(size_t)slot * heads + h] = aprod;
+    }
 }
 
 // per (segment, head), piece after piece: ws_state[slot] <- the state at the piece's start; the pool gets the last state
 __global__ void __launch_bounds__(256)
 decay_scan_combine_kernel(float* __restrict__ ws_state, const float* __restrict__ ws_decay, float* __restrict__ pool,
                           const int* __restrict__ state_in, const int* __restrict__ state_out,
-                          const int* __restrict__ seg_offsets, int heads, int hs, int piece) {
+                          const int* __restrict__ seg_offsets, int heads, int hs, int piece, int dk_c) {
     const int r = blockIdx.z, h = blockIdx.y, e = blockIdx.x * 256 + threadIdx.x;
     const int t0 = seg_offsets[r], len = seg_offsets[r + 1] - t0;
     if (len <= 0 || e >= hs) return;
@@ -553,7 +579,9 @@ decay_scan_combine_kernel(float* __restrict__ ws_state, const float* __restrict_
         float* at = ws_state + ((size_t)(base + p) * heads + h) * hs + e;
         const float local = *at;
         *at = S;
-        S = fmaf(ws_decay[(size_t)(base + p) * heads + h], S, local);
+        // (dk_c > 0: a product of decays per key channel, the fastest index of a head's state [dv][dk])
+        const float a = dk_c > 0 ? ws_decay[((size_t)(base + p) * heads + h) * dk_c + e % dk_c] : ws_decay[(size_t)(base + p) * heads + h];
+        S = fmaf(a, S, local);
     }
     pool[((size_t)state_out[r] * heads + h) * hs + e] = S;
 }
@@ -570,7 +598,7 @@ extern "C" int ilm_decay_scan(void* o, int o_stride, const void* q, const void* 
     ILM_REQUIRE(R > 0 && heads > 0 && dk > 0 && dv > 0 && T_ > 0, "decay_scan: bad sizes");
     if (decay_c != nullptr) {
         ILM_REQUIRE(decay_h == nullptr && decay_t == nullptr, "decay_scan: a decay per channel stands alone");
-        ILM_REQUIRE(piece == 0 && dc_stride >= heads * dk, "decay_scan: a decay per channel runs in one pass, rows of heads * dk");
+        ILM_REQUIRE(dc_stride >= heads * dk, "decay_scan: a decay per channel comes in rows of heads * dk");
     }
     ILM_REQUIRE(dk <= SC_NK * 64, "decay_scan: %d state entries a column, at most %d", dk, SC_NK * 64);
     ILM_REQUIRE(q_div > 0 && heads % q_div == 0, "decay_scan: %d heads do not divide into groups of %d", heads, q_div);
@@ -609,19 +637,26 @@ extern "C" int ilm_decay_scan(void* o, int o_stride, const void* q, const void* 
     const int cols = VT * (four ? 4 : 1), dkp = KP * SC_NK;
     int TB = 16;
     while (TB > 1 && (TB * dkp > 2048 || TB * cols > 2048)) TB >>= 1;
-    const size_t shm = (size_t)2 * TB * (2 * dkp + cols + 2) * sizeof(float);
+    const size_t shm = (size_t)2 * TB * ((decay_c != nullptr ? 3 : 2) * dkp + cols + 2) * sizeof(float);
+    ILM_REQUIRE(shm <= 64 * 1024, "decay_scan: a tile of %zu bytes does not fit LDS", shm);
     dim3 grid(four ? g4 : (dv + VT - 1) / VT, heads, slots);
 #define SCT_ARGS (float*)o, o_stride, (const float*)q, (const float*)k, qk_stride, q_div, (const float*)v, v_stride,             \
                  (const float*)decay_h, (const float*)decay_t, (const float*)kscale_t, (const float*)skip_h,                    \
                  (const int*)seg_offsets, heads, dk, dv, KP, R, piece, TB, (float*)ws_state, (float*)ws_decay
-    if (four) decay_scan_tiled_kernel<SC_LOCAL, 4><<<grid, 256, shm, stream>>>(SCT_ARGS);
+    if (decay_c != nullptr) {
+        if (four) decay_scan_tiled_kernel<SC_LOCAL, 4, true><<<grid, 256, shm, stream>>>(SCT_ARGS, (const float*)decay_c, dc_stride);
+        else decay_scan_tiled_kernel<SC_LOCAL, 1, true><<<grid, 256, shm, stream>>>(SCT_ARGS, (const float*)decay_c, dc_stride);
+    } else if (four) decay_scan_tiled_kernel<SC_LOCAL, 4><<<grid, 256, shm, stream>>>(SCT_ARGS);
     else decay_scan_tiled_kernel<SC_LOCAL, 1><<<grid, 256, shm, stream>>>(SCT_ARGS);
     ILM_LAUNCH_CHECK("decay_scan (local states)");
     decay_scan_combine_kernel<<<dim3((dk * dv + 255) / 256, heads, R), 256, 0, stream>>>(
         (float*)ws_state, (const float*)ws_decay, (float*)pool, (const int*)state_in, (const int*)state_out,
-        (const int*)seg_offsets, heads, dk * dv, piece);
+        (const int*)seg_offsets, heads, dk * dv, piece, decay_c != nullptr ? dk : 0);
     ILM_LAUNCH_CHECK("decay_scan (combine)");
-    if (four) decay_scan_tiled_kernel<SC_FROM, 4><<<grid, 256, shm, stream>>>(SCT_ARGS);
+    if (decay_c != nullptr) {
+        if (four) decay_scan_tiled_kernel<SC_FROM, 4, true><<<grid, 256, shm, stream>>>(SCT_ARGS, (const float*)decay_c, dc_stride);
+        else decay_scan_tiled_kernel<SC_FROM, 1, true><<<grid, 256, shm, stream>>>(SCT_ARGS, (const float*)decay_c, dc_stride);
+    } else if (four) decay_scan_tiled_kernel<SC_FROM, 4><<<grid, 256, shm, stream>>>(SCT_ARGS);
     else decay_scan_tiled_kernel<SC_FROM, 1><<<grid, 256, shm, stream>>>(SCT_ARGS);
     ILM_LAUNCH_CHECK("decay_scan (outputs)");
 #undef SCT_ARGS

@@ -1080,7 +1080,7 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, dk
     """S_t = a_t S_(t-1) + (b_t k_t) v_t^T, o_t = S_t^T q_t + skip_h v_t for every head of every segment, token by token,
     all in float32.  q, k: [T, groups*dk] (views with one row stride; head h reads group h // (heads/groups)), v [T, heads*dv];
     a per head (`decay_h` [heads]), per token (`decay_t` [T, heads]) or per token, head and key channel (`decay_c`
-    [T, heads*dk], float32 rows of one stride: S_t = diag(a_t) S_(t-1) + ..., always in one pass); b `kscale_t` [T, heads] or absent.  `pool`
+    [T, heads*dk], float32 rows of one stride: S_t = diag(a_t) S_(t-1) + ...); b `kscale_t` [T, heads] or absent.  `pool`
     [rows, heads, dv, dk] holds the states: segment r starts from row state_in[r] and leaves its state in row state_out[r].
     `max_len`: a bound on the segments' lengths known on the host; from SCAN_PIECE_FROM tokens on, segments are cut
     into pieces of SCAN_PIECE tokens that run side by side (two passes and a combination of the pieces' states; the
@@ -1115,12 +1115,11 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, dk
         raise KernelError("the recurrence takes a decay per head or per token, one of them")
     o = torch.empty((T, heads * dv), dtype=F32, device=v.device)
     piece, ws_state, ws_decay = 0, None, None
-    if (decay_c is None and SCAN_PIECE > 0 and max_len is not None and max_len >= SCAN_PIECE_FROM
-            and T // SCAN_PIECE + int(segments) <= 65535):
+    if SCAN_PIECE > 0 and max_len is not None and max_len >= SCAN_PIECE_FROM and T // SCAN_PIECE + int(segments) <= 65535:
         piece = SCAN_PIECE
         slots = T // piece + int(segments)
         ws_state = torch.empty((slots * heads * dv * dk,), dtype=F32, device=v.device)
-        ws_decay = torch.empty((slots * heads,), dtype=F32, device=v.device)
+        ws_decay = torch.empty((slots * heads * (dk if decay_c is not None else 1),), dtype=F32, device=v.device)
     _run("ilm_decay_scan", o.data_ptr(), o.stride(0), q.data_ptr(), k.data_ptr(), q.stride(0), heads // groups, v.data_ptr(),
          v.stride(0), _ptr(decay_h), _ptr(decay_t), _ptr(kscale_t), _ptr(skip_h), pool.data_ptr(), state_in.data_ptr(),
          state_out.data_ptr(), seg_offsets.data_ptr(), int(segments), heads, dk, dv, T, piece, _ptr(ws_state), _ptr(ws_decay),

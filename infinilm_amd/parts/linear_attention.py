@@ -157,7 +157,8 @@ class GatedLinearAttention(Mixer):
         alpha = kernels.sigmoid_root(z, self.tau, bias=self.a2.bias)
         f = kernels.linear_attention_inputs(rows, None, None, H, dk, dv, 0, "none", float(dk) ** -0.5)
         o = kernels.decay_scan(f[:, :H * dk], f[:, H * dk:2 * H * dk], f[:, 2 * H * dk:], H, dk, dv, H, view.pool,
-                               view.state_in, view.state_out, batch.seg_offsets, view.state_in.numel(), decay_c=alpha)
+                               view.state_in, view.state_out, batch.seg_offsets, view.state_in.numel(), decay_c=alpha,
+                               max_len=batch.max_q_len)
         y = kernels.group_norm_gate(o, self._norm_weight(), self.eps, H, gate=rows[:, g0:g0 + H * dv], gate_act="silu",
                                     out_dtype=self.dtype)
         return self.o_proj.forward(y, allow_parts=not self.whole_output)

@@ -163,11 +163,15 @@ def test_matrix_core_headmix_attention_equals_the_plain_kernel(nh, nkv, d, dv, w
     _close(each.view(T, nh, d), want, 2e-2, "the matrix-core kernel, token by token")
 
 
+@pytest.mark.parametrize("piece", [0, 4, 7])
 @pytest.mark.parametrize("heads,dk,dv", [(2, 16, 24), (3, 5, 3), (2, 128, 64), (1, 200, 40), (4, 64, 8)])
-def test_decay_per_channel_carries_states_over_launches(heads, dk, dv):
+def test_decay_per_channel_carries_states_over_launches(heads, dk, dv, piece, monkeypatch):
     """Three segments of unequal length in one launch, one from a zero state, two from the states an earlier launch left
-    in rows that are used again; every key channel with a decay of its own."""
+    in rows that are used again; every key channel with a decay of its own.  In one pass (`piece` 0) and with the segments
+    cut into pieces of 4 and of 7 tokens that run side by side."""
     from infinilm_amd import kernels
+    monkeypatch.setattr(kernels, "SCAN_PIECE", piece)
+    monkeypatch.setattr(kernels, "SCAN_PIECE_FROM", 1)
     g = torch.Generator().manual_seed(heads * 100 + dk)
     lens_a, lens_b = [7, 1, 19], [8, 33, 2]
     pool = torch.zeros((6, heads, dv, dk), device=DEV)
@@ -186,7 +190,7 @@ def test_decay_per_channel_carries_states_over_launches(heads, dk, dv):
             offs.append(offs[-1] + b - a)
         i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
         return kernels.decay_scan(cat(0), cat(1), cat(2), heads, dk, dv, heads, pool, i32(rows_in), i32(rows_out), i32(offs), len(spans),
-                                  decay_c=cat(3)).cpu(), offs
+                                  decay_c=cat(3), max_len=max(b - a for _, a, b in spans)).cpu(), offs
 
     o1, offs = launch([(r, 0, lens_a[r]) for r in range(3)], [0, 0, 0], [2, 4, 1])
     for r in range(3):
