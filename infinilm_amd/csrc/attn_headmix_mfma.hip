@@ -39,7 +39,7 @@ __device__ __forceinline__ uint32_t hx_pack(float lo, float hi) {
 // q' [T, nh, C, d] from q rows (head g at [g d, (g + 1) d)) and M [nh, nh] (null: the identity)
 // ------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)
-headmix_queries_kernel(bf16* __restrict__ qx, const bf16* __restrict__ q, const float* __restrict__ mix, int nh, int nkv, int d,
+headmix_queries_rows_kernel(bf16* __restrict__ qx, const bf16* __restrict__ q, const float* __restrict__ mix, int nh, int nkv, int d,
                        int q_stride) {
     extern __shared__ float qs[];
     const int t = blockIdx.x, per = nh / nkv;
@@ -58,12 +58,33 @@ headmix_queries_kernel(bf16* __restrict__ qx, const bf16* __restrict__ q, const 
     }
 }
 
+__global__ void __launch_bounds__(256)
+headmix_queries_kernel(bf16* __restrict__ qx, const bf16* __restrict__ q, const float* __restrict__ mix, int nh, int nkv, int d,
+                       int q_stride) {
+    // a block a (token, head h): its C d entries, each a sum over the heads of one group
+    const int t = blockIdx.x, h = blockIdx.y, per = nh / nkv;
+    const bf16* row = q + (size_t)t * q_stride;
+    bf16* dst = qx + ((size_t)t * nh + h) * nkv * d;
+    for (int idx = threadIdx.x; idx < nkv * d; idx += 256) {
+        const int e = idx % d, c = idx / d;
+        float a = 0.f;
+        for (int g = c * per; g < (c + 1) * per; ++g) {
+            const float m = mix != nullptr ? mix[h * nh + g] : (g == h ? 1.f : 0.f);
+            a = fmaf(m, to_f32(row[g * d + e]), a);
+        }
+        dst[idx] = from_f32<bf16>(a);
+    }
+}
+
+// few rows (decoded tokens): a block a (token, head); many: a block a token with its query heads in LDS
 extern "C" int ilm_headmix_queries(void* qx, const void* q, const void* mix, int T_, int nh, int nkv, int d, int q_stride,
                                    hipStream_t stream) {
-    ILM_REQUIRE(T_ > 0 && nh > 0 && nkv > 0 && nh % nkv == 0 && d > 0, "headmix_queries: bad sizes");
-    ILM_REQUIRE((size_t)nh * d * sizeof(float) <= 64 * 1024, "headmix_queries: %d heads of %d do not fit LDS", nh, d);
-    headmix_queries_kernel<<<T_, 256, (size_t)nh * d * sizeof(float), stream>>>((bf16*)qx, (const bf16*)q, (const float*)mix, nh, nkv, d,
-                                                                              q_stride);
+    ILM_REQUIRE(T_ > 0 && nh > 0 && nh <= 65535 && nkv > 0 && nh % nkv == 0 && d > 0, "headmix_queries: bad sizes");
+    if (T_ >= 256 && (size_t)nh * d * sizeof(float) <= 64 * 1024)
+        headmix_queries_rows_kernel<<<T_, 256, (size_t)nh * d * sizeof(float), stream>>>((bf16*)qx, (const bf16*)q, (const float*)mix, nh,
+                                                                                       nkv, d, q_stride);
+    else
+        headmix_queries_kernel<<<dim3(T_, nh), 256, 0, stream>>>((bf16*)qx, (const bf16*)q, (const float*)mix, nh, nkv, d, q_stride);
     ILM_LAUNCH_CHECK("headmix_queries");
     return 0;
 }
@@ -75,7 +96,7 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
                          const int* __restrict__ block_tables, const int* __restrict__ seg, const int* __restrict__ pos,
                          const int* __restrict__ tiles, int n_tiles, const int* __restrict__ singles,
                          const float* __restrict__ sink, int nh, int page, int max_blocks, int out_stride, float scale_log2e,
-                         int window) {
+                         int window, float* __restrict__ ws, int chunk_keys) {
     constexpr int D = D32 * 32, KROW = D + 8, VROW = HX_TK + 8;
     extern __shared__ __attribute__((aligned(16))) unsigned char hx_smem[];
     bf16* Ks = reinterpret_cast<bf16*>(hx_smem);                 // [NC][32][KROW]
@@ -123,7 +144,14 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
     }
     constexpr int KPIECES = NC * HX_TK * (D / 8), VPIECES = NC * D * (HX_TK / 8);
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
-    for (int kb = lo_first & ~(HX_TK - 1); kb <= p_last; kb += HX_TK) {
+    // chunk_keys > 0 (single tokens over long windows): this workgroup takes the keys of chunk blockIdx.z, counted from the
+    // first tile the token sees, and leaves a partial result (maximum, sum, unnormalised output) for the merge kernel
+    int kb_begin = lo_first & ~(HX_TK - 1), kb_end = p_last;
+    if (chunk_keys > 0) {
+        kb_begin += blockIdx.z * chunk_keys;
+        kb_end = min(p_last, kb_begin + chunk_keys - 1);
+    }
+    for (int kb = kb_begin; kb <= kb_end; kb += HX_TK) {
         const int pg = bt[kb / page];                            // (a tile lies on one page: the page size is a multiple of 32)
         const int off = kb % page;
         __syncthreads();                                         // the tile before this one has been read by every wave
@@ -198,6 +226,16 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
         float l = l_run[i];
         l += __shfl_xor(l, 16, 64);
         l += __shfl_xor(l, 32, 64);
+        if (chunk_keys > 0) {
+            if (r == 0) {      // (a single token: column 0)
+                float* dst = ws + (((size_t)blockIdx.x * gridDim.z + blockIdx.z) * nh + head[i]) * (D + 4);
+#pragma unroll
+                for (int b = 0; b < 2 * D32; ++b)
+                    *reinterpret_cast<float4*>(dst + b * 16 + g4 * 4) = make_float4(O[i][b][0], O[i][b][1], O[i][b][2], O[i][b][3]);
+                if (g4 == 0) { dst[D] = m_run[i]; dst[D + 1] = l; }
+            }
+            continue;
+        }
         if (sink != nullptr) l += __builtin_amdgcn_exp2f(sink[head[i]] * 1.4426950408889634f - m_run[i]);
         const float inv = 1.0f / l;
         if (tok_ok) {
@@ -211,6 +249,27 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
     }
 }
 
+// the chunks' partial results of a single token and head folded in order, the sink's term, the division
+__global__ void __launch_bounds__(128)
+attn_headmix_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws, const int* __restrict__ singles,
+                          const float* __restrict__ sink, int nh, int D, int nz, int out_stride) {
+    const int item = blockIdx.x, h = blockIdx.y, e = threadIdx.x;
+    const int t = singles != nullptr ? singles[item] : item;
+    if (t < 0 || e >= D) return;
+    float M = HX_NEG, L = 0.f, A = 0.f;
+    for (int z = 0; z < nz; ++z) {
+        const float* src = ws + (((size_t)item * nz + z) * nh + h) * (D + 4);
+        const float m = src[D], l = src[D + 1];
+        const float Mn = fmaxf(M, m);
+        const float a = __builtin_amdgcn_exp2f(M - Mn), b = __builtin_amdgcn_exp2f(m - Mn);
+        L = fmaf(L, a, l * b);
+        A = fmaf(A, a, src[e] * b);
+        M = Mn;
+    }
+    if (sink != nullptr) L += __builtin_amdgcn_exp2f(sink[h] * 1.4426950408889634f - M);
+    out[(size_t)t * out_stride + (size_t)h * D + e] = from_f32<bf16>(A / L);
+}
+
 extern "C" int ilm_attn_headmix_mfma_ok(int nh, int nkv, int d, int page) {
     return nh > 0 && nkv > 0 && nh % nkv == 0 && (nkv == 1 || nkv == 2 || nkv == 4) && d % 32 == 0 && d >= 32 && d <= 128 &&
            page % HX_TK == 0;
@@ -221,7 +280,12 @@ extern "C" int ilm_attn_headmix_mfma_ok(int nh, int nkv, int d, int page) {
 extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, const void* vc, const void* block_tables,
                                      const void* seg, const void* pos, const void* tiles, int n_tiles, const void* singles,
                                      int n_singles, const void* sink, int nh, int nkv, int d, int page, int max_blocks,
-                                     int out_stride, float scale, int window, hipStream_t stream) {
+                                     int out_stride, float scale, int window, void* ws, int nz, int chunk_keys,
+                                     hipStream_t stream) {
+    // ws != null (single tokens only): nz chunks of chunk_keys keys a token, float [n_singles][nz][nh][d + 4]
+    ILM_REQUIRE(ws == nullptr || (n_tiles == 0 && nz >= 1 && nz <= 65535 && chunk_keys > 0 && chunk_keys % HX_TK == 0),
+                "attn_headmix_mfma: chunks are for single tokens, in multiples of %d keys", HX_TK);
+    if (ws == nullptr) { nz = 1; chunk_keys = 0; }
     ILM_REQUIRE(n_tiles >= 0 && n_singles >= 0 && n_tiles + n_singles > 0 && max_blocks > 0, "attn_headmix_mfma: bad sizes");
     ILM_REQUIRE(ilm_attn_headmix_mfma_ok(nh, nkv, d, page), "attn_headmix_mfma: %d heads in %d groups of %d, pages of %d", nh, nkv, d, page);
     ILM_REQUIRE(out_stride % 4 == 0 && ((uintptr_t)out & 7) == 0 && ((uintptr_t)qx & 15) == 0 && ((uintptr_t)kc & 15) == 0 &&
@@ -235,11 +299,11 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
             hipError_t e_ = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm);       \
             ILM_REQUIRE(e_ == hipSuccess, "attn_headmix_mfma: %d bytes of LDS refused: %s", shm, hipGetErrorString(e_));   \
         }                                                                                                                  \
-        dim3 grid(n_tiles + n_singles, (nh + 4 * HPW_ - 1) / (4 * HPW_));                                                  \
+        dim3 grid(n_tiles + n_singles, (nh + 4 * HPW_ - 1) / (4 * HPW_), nz);                                              \
         kern<<<grid, 256, shm, stream>>>((bf16*)out, (const bf16*)qx, (const bf16*)kc, (const bf16*)vc,                    \
                                          (const int*)block_tables, (const int*)seg, (const int*)pos, (const int*)tiles,    \
                                          n_tiles, (const int*)singles, (const float*)sink, nh, page, max_blocks,           \
-                                         out_stride, scale_log2e, window);                                                 \
+                                         out_stride, scale_log2e, window, (float*)ws, chunk_keys);                         \
     }
 #define HX_BY_NC(D32_)                                                      \
     switch (nkv) {                                                          \
@@ -256,5 +320,10 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
 #undef HX_BY_NC
 #undef HX_LAUNCH
     ILM_LAUNCH_CHECK("attn_headmix_mfma");
+    if (ws != nullptr) {
+        attn_headmix_merge_kernel<<<dim3(n_singles, nh), 128, 0, stream>>>((bf16*)out, (const float*)ws, (const int*)singles,
+                                                                           (const float*)sink, nh, d, nz, out_stride);
+        ILM_LAUNCH_CHECK("attn_headmix_mfma (merge)");
+    }
     return 0;
 }

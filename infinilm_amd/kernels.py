@@ -1356,7 +1356,8 @@ def qkv_norm_rope_kvwrite(qkv: torch.Tensor, positions: torch.Tensor, freq: Opti
 def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
                       seg_of_token: torch.Tensor, positions: torch.Tensor, nh: int, nkv: int, d: int, dv: int, scale: float,
                       window: int = 0, mix: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
-                      tiles: Optional[torch.Tensor] = None, single_rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      tiles: Optional[torch.Tensor] = None, single_rows: Optional[torch.Tensor] = None,
+                      max_total_len: Optional[int] = None) -> torch.Tensor:
     """Attention of every token over its request's cached keys (its last `window` positions, or all) where the scaled
     scores of the heads are mixed before the softmax, s_h = sum_g mix[h, g] raw_g (`mix` float32 [nh, nh] or None),
     and every head's denominator holds one more term exp(sink[h]) (`sink` float32 [nh] or None).  q, caches, block
@@ -1393,9 +1394,28 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
             if single_rows is not None and single_rows.numel() > 0:
                 _i32(single_rows, "single_rows")
                 rows, n_single = single_rows, single_rows.numel()
+        # single tokens over long windows (decoding): the keys in chunks over more workgroups, and a merge.  The chunks are
+        # sized by bounded numbers (rows as recorded steps round them, the block table's width), so an eager step and its
+        # recording cut alike.
+        ws, nz, chunk = None, 1, 0
+        if n_tiles == 0:
+            span = block_tables.shape[1] * page
+            if max_total_len is not None:
+                span = min(span, bound_pages(-(-int(max_total_len) // page)) * page)
+            if window > 0:
+                span = min(span, int(window) + 32)
+            passes = -(-nh // (4 * (4 if nkv * (d // 32) <= 4 else 2 if nkv * (d // 32) <= 8 else 1)))
+            want = max(1, (4 * _num_cus(q.device)) // max(1, bound_rows(n_single) * passes))
+            chunk = max(128, -(-(-(-span // want)) // 32) * 32)
+            nz = -(-span // chunk)
+            if nz > 1:
+                ws = torch.empty((n_single * nz * nh * (d + 4),), dtype=F32, device=q.device)
+            else:
+                nz, chunk = 1, 0
         _run("ilm_attn_headmix_mfma", out.data_ptr(), qx.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
              seg_of_token.data_ptr(), positions.data_ptr(), _ptr(tiles) if n_tiles else None, n_tiles, _ptr(rows), n_single,
-             _ptr(sink), nh, nkv, d, page, block_tables.shape[1], out.stride(0), float(scale), int(window), _stream())
+             _ptr(sink), nh, nkv, d, page, block_tables.shape[1], out.stride(0), float(scale), int(window), _ptr(ws), nz, chunk,
+             _stream())
         return out
     _run("ilm_attn_headmix", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
          seg_of_token.data_ptr(), positions.data_ptr(), None, T, _ptr(mix), _ptr(sink), nh, nkv, d, int(dv), page,
