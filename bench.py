@@ -195,12 +195,13 @@ def compare_designs(args) -> dict:
                             4.0 * T * T / 2 * heads * d / us(rep_p, "ilm_attn_tile") / FLOP_PEAK["bf16"], 4)
                     if name == "pugavik":
                         win = 1024
-                        if us(rep_d, "ilm_attn_headmix"):
+                        hm = "ilm_attn_headmix_mfma" if "ilm_attn_headmix_mfma" in rep_d else "ilm_attn_headmix"
+                        if us(rep_d, hm):
                             seen = min(ctx, win)
-                            share["attn_headmix decode (window's cache read / HBM peak)"] = round(64 * seen * kvb / us(rep_d, "ilm_attn_headmix") / HBM_PEAK, 4)
+                            share["mixed-heads attention decode (window's cache read / HBM peak)"] = round(64 * seen * kvb / us(rep_d, hm) / HBM_PEAK, 4)
                             pairs = sum(min(i + 1, win) for i in range(T))
-                            share["attn_headmix prefill ((4 d + 2 heads) flops a visible key and head / float32 vector peak)"] = round(
-                                (4.0 * d + 2.0 * heads) * pairs * heads / us(rep_p, "ilm_attn_headmix") / FLOP_PEAK["fp32"], 4)
+                            share["mixed-heads attention prefill (4 d flops a visible key and head / bf16 matrix peak)"] = round(
+                                4.0 * d * pairs * heads / us(rep_p, hm) / FLOP_PEAK["bf16"], 4)
                         gstate = heads * (d // 2) * d * 4
                         if us(rep_d, "ilm_decay_scan"):
                             share["decay_scan (decay per channel) decode (state read + written / HBM peak)"] = round(64 * 2 * gstate / us(rep_d, "ilm_decay_scan") / HBM_PEAK, 4)
