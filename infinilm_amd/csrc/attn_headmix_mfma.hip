@@ -9,13 +9,16 @@
 // between heads; for many groups the plain kernel's explicit mixing does less work.
 //
 // A workgroup = one item (a tile of up to 8 consecutive tokens of a request, or a single token) x one pass of 4 HPW
-// heads; its 4 waves take HPW heads each.  Keys go by in tiles of 32 aligned to the absolute key index; K [group][key][d]
+// heads; its 4 waves take HPW heads each.  Keys go by in tiles of 32 or 64 aligned to the absolute key index; K [group][key][d]
 // and V [group][d][key] of a tile pass through LDS once for all heads of the pass.  Per head and tile:
-//   S^T [32 keys x 16 tokens] = K q'^T        (v_mfma_f32_16x16x32_bf16: A = K rows, B = q' rows; lane (r, g4) gets
+//   S^T [keys x 16 tokens] = K q'^T           (v_mfma_f32_16x16x32_bf16: A = K rows, B = q' rows; lane (r, g4) gets
 //                                              keys 4 g4 .. 4 g4 + 3 of each 16-key half for token r)
 //   running maximum, sum and weights per token (a token's keys lie in 4 lanes x 8 registers)
 //   O^T [d x 16 tokens] += V^T P^T            (A = V rows [d][key], B = the weights as they lie in the registers: the k index
 //                                              of this product is a fixed permutation of the keys, the same for A and B)
+// Scores, maxima, exponentials and sums are float; the weights enter the second product as two bfloat16 terms (hi + lo).
+// Without a mixing matrix and with one group the mixed queries are the queries themselves: the kernel then is a plain flash
+// attention whose weights stay float, for mixers that want them so.
 // A token's result depends on its position and its request's cache alone: keys outside its window weigh exactly zero
 // and leave its running maximum alone, whatever other tokens share the tile.
 #include "common.h"
@@ -23,7 +26,6 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 hx_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float hx_f32x4;
 
-#define HX_TK 32
 #define HX_TT 8            // tokens a tile at most (the step's lists hold tiles of up to 8)
 #define HX_NEG (-1.0e30f)
 
@@ -90,17 +92,19 @@ extern "C" int ilm_headmix_queries(void* qx, const void* q, const void* mix, int
 }
 
 // ------------------------------------------------------------------------------------------
-template <int D32, int NC, int HPW>
+// TK: keys a tile (32; tiles of 64 halve the rounds of loads and barriers and measured slower: 437 against 374 us a
+// prompt step at 32 heads of 128, more LDS a workgroup and fewer workgroups a unit)
+template <int D32, int NC, int HPW, int TK>
 __global__ void __launch_bounds__(256)
 attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                          const int* __restrict__ block_tables, const int* __restrict__ seg, const int* __restrict__ pos,
                          const int* __restrict__ tiles, int n_tiles, const int* __restrict__ singles,
                          const float* __restrict__ sink, int nh, int page, int max_blocks, int out_stride, float scale_log2e,
                          int window, float* __restrict__ ws, int chunk_keys) {
-    constexpr int D = D32 * 32, KROW = D + 8, VROW = HX_TK + 8;
+    constexpr int D = D32 * 32, KROW = D + 8, VROW = TK + 8, NS = TK / 16, NP = TK / 32;
     extern __shared__ __attribute__((aligned(16))) unsigned char hx_smem[];
     bf16* Ks = reinterpret_cast<bf16*>(hx_smem);                 // [NC][32][KROW]
-    bf16* Vs = Ks + NC * HX_TK * KROW;                           // [NC][D][VROW]
+    bf16* Vs = Ks + NC * TK * KROW;                              // [NC][D][VROW]
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, g4 = lane >> 4, wave = tid >> 6;
     int t0, ntok;
     if ((int)blockIdx.x < n_tiles) {
@@ -142,52 +146,54 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
         m_run[i] = HX_NEG;
         l_run[i] = 0.f;
     }
-    constexpr int KPIECES = NC * HX_TK * (D / 8), VPIECES = NC * D * (HX_TK / 8);
+    constexpr int KPIECES = NC * TK * (D / 8), VPIECES = NC * D * (TK / 8);
     const uint4 zero4 = make_uint4(0u, 0u, 0u, 0u);
     // chunk_keys > 0 (single tokens over long windows): this workgroup takes the keys of chunk blockIdx.z, counted from the
     // first tile the token sees, and leaves a partial result (maximum, sum, unnormalised output) for the merge kernel
-    int kb_begin = lo_first & ~(HX_TK - 1), kb_end = p_last;
+    int kb_begin = lo_first & ~(TK - 1), kb_end = p_last;
     if (chunk_keys > 0) {
         kb_begin += blockIdx.z * chunk_keys;
         kb_end = min(p_last, kb_begin + chunk_keys - 1);
     }
-    for (int kb = kb_begin; kb <= kb_end; kb += HX_TK) {
+    for (int kb = kb_begin; kb <= kb_end; kb += TK) {
         const int pg = bt[kb / page];                            // (a tile lies on one page: the page size is a multiple of 32)
         const int off = kb % page;
         __syncthreads();                                         // the tile before this one has been read by every wave
         for (int pc = tid; pc < KPIECES; pc += 256) {
-            const int c = pc / (HX_TK * (D / 8)), rest = pc % (HX_TK * (D / 8)), key = rest / (D / 8), piece = rest % (D / 8);
+            const int c = pc / (TK * (D / 8)), rest = pc % (TK * (D / 8)), key = rest / (D / 8), piece = rest % (D / 8);
             uint4 v = zero4;
             if (pg >= 0) v = *reinterpret_cast<const uint4*>(kc + (((size_t)pg * NC + c) * page + off + key) * D + piece * 8);
-            *reinterpret_cast<uint4*>(Ks + (c * HX_TK + key) * KROW + piece * 8) = v;
+            *reinterpret_cast<uint4*>(Ks + (c * TK + key) * KROW + piece * 8) = v;
         }
         for (int pc = tid; pc < VPIECES; pc += 256) {
-            const int c = pc / (D * (HX_TK / 8)), rest = pc % (D * (HX_TK / 8)), row = rest / (HX_TK / 8), piece = rest % (HX_TK / 8);
+            const int c = pc / (D * (TK / 8)), rest = pc % (D * (TK / 8)), row = rest / (TK / 8), piece = rest % (TK / 8);
             uint4 v = zero4;
             if (pg >= 0) v = *reinterpret_cast<const uint4*>(vc + (((size_t)pg * NC + c) * D + row) * page + off + piece * 8);
             *reinterpret_cast<uint4*>(Vs + (c * D + row) * VROW + piece * 8) = v;
         }
         __syncthreads();
+        // head by head (a version that read every key and value fragment from LDS once for all heads of a wave kept more
+        // registers live and measured slower: 455 against 374 us a prompt step at 32 heads of 128)
 #pragma unroll
         for (int i = 0; i < HPW; ++i) {
             if (!head_ok[i]) continue;                           // (uniform over the wave)
-            hx_f32x4 S[2];
+            hx_f32x4 S[NS];
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
+            for (int s = 0; s < NS; ++s) {
                 S[s] = hx_f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int c = 0; c < NC; ++c)
 #pragma unroll
                     for (int ks = 0; ks < D32; ++ks) {
-                        const uint4 a = *reinterpret_cast<const uint4*>(Ks + (c * HX_TK + s * 16 + r) * KROW + ks * 32 + g4 * 8);
+                        const uint4 a = *reinterpret_cast<const uint4*>(Ks + (c * TK + s * 16 + r) * KROW + ks * 32 + g4 * 8);
                         S[s] = hx_mfma(a, qf[i][c][ks], S[s]);
                     }
             }
             // this lane: token r, keys kb + 16 s + 4 g4 + j
-            float sc[8];
+            float sc[4 * NS];
             float mx = HX_NEG;
 #pragma unroll
-            for (int s = 0; s < 2; ++s)
+            for (int s = 0; s < NS; ++s)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int key = kb + s * 16 + g4 * 4 + j;
@@ -199,24 +205,40 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
             const float m_new = fmaxf(m_run[i], mx);
             const float corr = __builtin_amdgcn_exp2f(m_run[i] - m_new);
-            float pw[8], sum = 0.f;
+            float pw[4 * NS], sum = 0.f;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
+            for (int j = 0; j < 4 * NS; ++j) {
                 pw[j] = sc[j] > 0.5f * HX_NEG ? __builtin_amdgcn_exp2f(sc[j] - m_new) : 0.f;
                 sum += pw[j];
             }
             l_run[i] = l_run[i] * corr + sum;                    // (this lane's share; the four lanes of a token are summed at the end)
             m_run[i] = m_new;
-            const uint4 pb = make_uint4(hx_pack(pw[0], pw[1]), hx_pack(pw[2], pw[3]), hx_pack(pw[4], pw[5]), hx_pack(pw[6], pw[7]));
+            // the float weights enter the second product as two bfloat16 terms (the rounded weight and what the rounding
+            // left), so 16 bits of each weight count instead of 8; a product takes 32 keys: subtiles 2 u and 2 u + 1
+            uint4 pb[NP], pb_lo[NP];
+#pragma unroll
+            for (int u = 0; u < NP; ++u) {
+                float pl[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) pl[j] = pw[8 * u + j] - to_f32(from_f32<bf16>(pw[8 * u + j]));
+                pb[u] = make_uint4(hx_pack(pw[8 * u], pw[8 * u + 1]), hx_pack(pw[8 * u + 2], pw[8 * u + 3]), hx_pack(pw[8 * u + 4], pw[8 * u + 5]),
+                                   hx_pack(pw[8 * u + 6], pw[8 * u + 7]));
+                pb_lo[u] = make_uint4(hx_pack(pl[0], pl[1]), hx_pack(pl[2], pl[3]), hx_pack(pl[4], pl[5]), hx_pack(pl[6], pl[7]));
+            }
             const int c_h = head[i] / per;
 #pragma unroll
             for (int b = 0; b < 2 * D32; ++b) {
                 const bf16* vrow = Vs + (c_h * D + b * 16 + r) * VROW;
-                const uint2 v0 = *reinterpret_cast<const uint2*>(vrow + g4 * 4);          // keys 4 g4 .. + 3
-                const uint2 v1 = *reinterpret_cast<const uint2*>(vrow + 16 + g4 * 4);     // keys 16 + 4 g4 .. + 3
                 hx_f32x4 o = O[i][b];
                 o[0] *= corr; o[1] *= corr; o[2] *= corr; o[3] *= corr;
-                O[i][b] = hx_mfma(make_uint4(v0.x, v0.y, v1.x, v1.y), pb, o);
+#pragma unroll
+                for (int u = 0; u < NP; ++u) {
+                    const uint2 v0 = *reinterpret_cast<const uint2*>(vrow + 32 * u + g4 * 4);          // keys 32 u + 4 g4 .. + 3
+                    const uint2 v1 = *reinterpret_cast<const uint2*>(vrow + 32 * u + 16 + g4 * 4);     // keys 32 u + 16 + 4 g4 .. + 3
+                    const uint4 va = make_uint4(v0.x, v0.y, v1.x, v1.y);
+                    o = hx_mfma(va, pb_lo[u], hx_mfma(va, pb[u], o));
+                }
+                O[i][b] = o;
             }
         }
     }
@@ -272,7 +294,7 @@ attn_headmix_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws, 
 
 extern "C" int ilm_attn_headmix_mfma_ok(int nh, int nkv, int d, int page) {
     return nh > 0 && nkv > 0 && nh % nkv == 0 && (nkv == 1 || nkv == 2 || nkv == 4) && d % 32 == 0 && d >= 32 && d <= 128 &&
-           page % HX_TK == 0;
+           page % 32 == 0;
 }
 
 // qx [T, nh, nkv, d] from ilm_headmix_queries; tiles [n_tiles, 2] = (first row, count <= 8) and n_singles single rows
@@ -283,8 +305,8 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
                                      int out_stride, float scale, int window, void* ws, int nz, int chunk_keys,
                                      hipStream_t stream) {
     // ws != null (single tokens only): nz chunks of chunk_keys keys a token, float [n_singles][nz][nh][d + 4]
-    ILM_REQUIRE(ws == nullptr || (n_tiles == 0 && nz >= 1 && nz <= 65535 && chunk_keys > 0 && chunk_keys % HX_TK == 0),
-                "attn_headmix_mfma: chunks are for single tokens, in multiples of %d keys", HX_TK);
+    ILM_REQUIRE(ws == nullptr || (n_tiles == 0 && nz >= 1 && nz <= 65535 && chunk_keys > 0 && chunk_keys % 64 == 0),
+                "attn_headmix_mfma: chunks are for single tokens, in multiples of 64 keys");
     if (ws == nullptr) { nz = 1; chunk_keys = 0; }
     ILM_REQUIRE(n_tiles >= 0 && n_singles >= 0 && n_tiles + n_singles > 0 && max_blocks > 0, "attn_headmix_mfma: bad sizes");
     ILM_REQUIRE(ilm_attn_headmix_mfma_ok(nh, nkv, d, page), "attn_headmix_mfma: %d heads in %d groups of %d, pages of %d", nh, nkv, d, page);
@@ -292,9 +314,11 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
                 ((uintptr_t)vc & 15) == 0, "attn_headmix_mfma: rows must be 16-byte / 8-byte aligned");
     const float scale_log2e = scale * 1.4426950408889634f;
 #define HX_LAUNCH(D32_, NC_, HPW_)                                                                                         \
+    HX_LAUNCH_TK(D32_, NC_, HPW_, 32)
+#define HX_LAUNCH_TK(D32_, NC_, HPW_, TK_)                                                                                 \
     {                                                                                                                      \
-        auto kern = attn_headmix_mfma_kernel<D32_, NC_, HPW_>;                                                             \
-        const int shm = NC_ * HX_TK * (D32_ * 32 + 8) * 2 + NC_ * D32_ * 32 * (HX_TK + 8) * 2;                             \
+        auto kern = attn_headmix_mfma_kernel<D32_, NC_, HPW_, TK_>;                                                        \
+        const int shm = NC_ * TK_ * (D32_ * 32 + 8) * 2 + NC_ * D32_ * 32 * (TK_ + 8) * 2;                                 \
         if (shm > 48 * 1024) {                                                                                             \
             hipError_t e_ = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm);       \
             ILM_REQUIRE(e_ == hipSuccess, "attn_headmix_mfma: %d bytes of LDS refused: %s", shm, hipGetErrorString(e_));   \
@@ -307,8 +331,8 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
     }
 #define HX_BY_NC(D32_)                                                      \
     switch (nkv) {                                                          \
-        case 1: HX_LAUNCH(D32_, 1, 4) break;                                \
-        case 2: if (D32_ <= 2) HX_LAUNCH(D32_, 2, 4) else HX_LAUNCH(D32_, 2, 2) break; \
+        case 1: if (D32_ <= 2) HX_LAUNCH(D32_, 1, 4) else HX_LAUNCH(D32_, 1, 1) break; \
+        case 2: if (D32_ <= 2) HX_LAUNCH(D32_, 2, 4) else HX_LAUNCH(D32_, 2, 1) break; \
         default: if (D32_ <= 2) HX_LAUNCH(D32_, 4, 2) else HX_LAUNCH(D32_, 4, 1) break; \
     }
     switch (d / 32) {
@@ -319,6 +343,7 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
     }
 #undef HX_BY_NC
 #undef HX_LAUNCH
+#undef HX_LAUNCH_TK
     ILM_LAUNCH_CHECK("attn_headmix_mfma");
     if (ws != nullptr) {
         attn_headmix_merge_kernel<<<dim3(n_singles, nh), 128, 0, stream>>>((bf16*)out, (const float*)ws, (const int*)singles,

@@ -677,9 +677,11 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     seg_of_token: torch.Tensor, positions: torch.Tensor, nh: int, nkv: int, d: int,
                     scale: float, window: int = 0, max_total_len: Optional[int] = None,
                     tiles: Optional[torch.Tensor] = None, single_rows: Optional[torch.Tensor] = None,
-                    softcap: float = 0.0) -> torch.Tensor:
+                    softcap: float = 0.0, float_weights: bool = False) -> torch.Tensor:
     """Attention of every token over its request's cached keys up to its own position.
     `softcap` > 0: scaled scores pass through softcap * tanh(score / softcap) before the softmax.
+    `float_weights`: the softmax weights stay float32 in the second product (the bfloat16 matrix-core kernels round them:
+    they are passed over, the plain kernel runs).
 
     q: rows of T tokens in which head h lies at [h*d, (h+1)*d) (a view into the fused projection is
     fine); caches as the cache manager lays them out; block_tables [R, max_blocks]; `max_total_len`: an
@@ -700,8 +702,8 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     if seg_of_token.numel() != T or positions.numel() != T or block_tables.dim() != 2:
         raise KernelError("per-token metadata does not match the number of tokens")
     out = torch.empty((T, nh * d), dtype=q.dtype, device=q.device)
-    if (q.dtype == BF16 and not FORCE_BASIC and d % 16 == 0 and d <= 128 and page % 16 == 0 and q.stride(0) % 8 == 0
-            and max_total_len is not None):
+    if (q.dtype == BF16 and not FORCE_BASIC and not float_weights and d % 16 == 0 and d <= 128 and page % 16 == 0
+            and q.stride(0) % 8 == 0 and max_total_len is not None):
         n_single = T
         rows = None
         if tiles is not None and tiles.numel() > 0:
@@ -1319,6 +1321,11 @@ def add_layernorm(residual: torch.Tensor, addends, weight: Optional[torch.Tensor
 
 
 # ---- attention with scores mixed over the heads ----------------------------------------------------
+def headmix_mfma_ok(nh: int, nkv: int, d: int, page: int, dtype: torch.dtype) -> bool:
+    """Whether `headmix_attention` runs its matrix-core kernel for these sizes."""
+    return bool(dtype == BF16 and not FORCE_BASIC and USE_HEADMIX_MFMA and _lib().ilm_attn_headmix_mfma_ok(nh, nkv, d, page))
+
+
 USE_HEADMIX_MFMA = os.environ.get("INFINILM_AMD_HEADMIX_MFMA", "1") == "1"   # 0: always the plain kernel
 
 
@@ -1360,7 +1367,8 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       max_total_len: Optional[int] = None) -> torch.Tensor:
     """Attention of every token over its request's cached keys (its last `window` positions, or all) where the scaled
     scores of the heads are mixed before the softmax, s_h = sum_g mix[h, g] raw_g (`mix` float32 [nh, nh] or None),
-    and every head's denominator holds one more term exp(sink[h]) (`sink` float32 [nh] or None).  q, caches, block
+    and every head's denominator holds one more term exp(sink[h]) (`sink` float32 [nh] or None); with neither it is the
+    attention of `paged_attention` with its weights kept in float32 up to the second product.  q, caches, block
     tables as for `paged_attention`; `dv`: the entries of a value head that count.  `tiles` [n, 2] = (first row, count <=
     ATT_TILE_TOKENS) lists runs of consecutive tokens of one request and `single_rows` the remaining rows (without them
     every token is served on its own); the matrix-core kernel (bfloat16, heads of 32 to 128 in steps of 32, 1, 2 or 4
@@ -1385,8 +1393,11 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     if (q.dtype == BF16 and not FORCE_BASIC and USE_HEADMIX_MFMA and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0
             and _lib().ilm_attn_headmix_mfma_ok(nh, nkv, d, page)):
         # the mixing carried into the queries, then a flash attention on the matrix cores
-        qx = torch.empty((T, nh, nkv, d), dtype=BF16, device=q.device)
-        _run("ilm_headmix_queries", qx.data_ptr(), q.data_ptr(), _ptr(mix), T, nh, nkv, d, q.stride(0), _stream())
+        if mix is None and nkv == 1 and q.stride(0) == nh * d:
+            qx = q        # one group and no mixing: the mixed queries are the queries
+        else:
+            qx = torch.empty((T, nh, nkv, d), dtype=BF16, device=q.device)
+            _run("ilm_headmix_queries", qx.data_ptr(), q.data_ptr(), _ptr(mix), T, nh, nkv, d, q.stride(0), _stream())
         n_tiles, n_single, rows = 0, T, None
         if tiles is not None and tiles.numel() > 0:
             _i32(tiles, "tiles")
@@ -1403,10 +1414,11 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
             if max_total_len is not None:
                 span = min(span, bound_pages(-(-int(max_total_len) // page)) * page)
             if window > 0:
-                span = min(span, int(window) + 32)
-            passes = -(-nh // (4 * (4 if nkv * (d // 32) <= 4 else 2 if nkv * (d // 32) <= 8 else 1)))
+                span = min(span, int(window) + 64)
+            hpw = 1 if d > 64 else (2 if nkv == 4 else 4)      # heads a wave, as the kernel's launcher picks them
+            passes = -(-nh // (4 * hpw))
             want = max(1, (4 * _num_cus(q.device)) // max(1, bound_rows(n_single) * passes))
-            chunk = max(128, -(-(-(-span // want)) // 32) * 32)
+            chunk = max(128, -(-(-(-span // want)) // 64) * 64)
             nz = -(-span // chunk)
             if nz > 1:
                 ws = torch.empty((n_single * nz * nh * (d + 4),), dtype=F32, device=q.device)

@@ -10,8 +10,9 @@ The cache holds c and the rotated key part only.  The step runs the absorbed for
 into the latent space (W_uk,h^T q_h, a product per head), so the scores are dot products of rows of kv_rank + rot_dim
 entries against one cached key row per token, the attention's values are the latent rows themselves, and W_uv,h is
 applied to the head's result afterwards.  That makes it an attention with one key/value head of
-d = kv_rank + rot_dim (rounded up to a multiple of 16) entries, which the paged attention kernels serve: the key row is
-[c | rotated part | zeros], the value row [c | zeros].  Rotation: entry pairs (2i, 2i + 1), angle p * theta^(-2i/rot_dim),
+d = kv_rank + rot_dim (rounded up to a multiple of 32, of 16 beyond 128) entries: the key row is [c | rotated part | zeros],
+the value row [c | zeros], and the attention is the kernels' that keep the softmax weights in float32 (the matrix-core kernel
+of `kernels.headmix_attention` without mixing and sink, or the plain paged kernel).  Rotation: entry pairs (2i, 2i + 1), angle p * theta^(-2i/rot_dim),
 formed in float32 in the kernel.
 """
 from __future__ import annotations
@@ -38,7 +39,10 @@ class LatentAttention(Mixer):
         self.H, self.dn, self.dr, self.dv, self.rank = int(heads), int(head_dim), int(rotary_dim), int(value_dim), int(kv_rank)
         if self.dr % 2:
             raise ValueError(f"{self.dr} rotated entries must be even")
-        self.d = -(-(self.rank + self.dr) // 16) * 16           # the head size the attention runs
+        # the head size the attention runs: the next multiple of 32 up to 128 (the matrix-core kernel with float weights), of
+        # 16 beyond
+        need = self.rank + self.dr
+        self.d = -(-need // 32) * 32 if need <= 128 else -(-need // 16) * 16
         self.scale, self.eps, self.window = float(scale), float(eps), int(window)
         self.whole_output = bool(whole_output)
         self.dtype = ctx.dtype
@@ -68,8 +72,17 @@ class LatentAttention(Mixer):
         kernels.latent_prep(rows, qx, batch.positions, self.freq, self.norm_w, view.k, view.v, view.slots, H, dn, dr, rank, d, self.eps)
         q_plain = rows[:, :H * (dn + dr)].view(T, H, dn + dr)[:, :, :dn]
         kernels.head_gemm(q_plain, self.uk.weight.view(H, dn, rank), qx[:, :, :rank])          # q_h^T W_uk,h
-        o = kernels.paged_attention(qx.view(T, H * d), view.k, view.v, view.block_tables, batch.seg_of_token, batch.positions,
-                                    H, 1, d, self.scale, self.window, batch.max_total_len, batch.att_tiles, batch.att_single_rows)
+        # bfloat16: the kernels that keep the softmax weights float32 up to the second product (the matrix-core kernel with
+        # its two-term weights where the sizes fit, else the plain one); float32: everything is float anyway
+        q2 = qx.view(T, H * d)
+        if rows.dtype == torch.bfloat16 and kernels.headmix_mfma_ok(H, 1, d, view.page_size, rows.dtype):
+            o = kernels.headmix_attention(q2, view.k, view.v, view.block_tables, batch.seg_of_token, batch.positions, H, 1, d, rank,
+                                          self.scale, self.window, tiles=batch.att_tiles, single_rows=batch.att_single_rows,
+                                          max_total_len=batch.max_total_len)
+        else:
+            o = kernels.paged_attention(q2, view.k, view.v, view.block_tables, batch.seg_of_token, batch.positions, H, 1, d,
+                                        self.scale, self.window, batch.max_total_len, batch.att_tiles, batch.att_single_rows,
+                                        float_weights=True)
         y = torch.empty((T, H, dv), dtype=rows.dtype, device=rows.device)
         kernels.head_gemm(o.view(T, H, d)[:, :, :rank], self.uv.weight.view(H, dv, rank).transpose(1, 2), y)   # W_uv,h (sum_j p_j c_j)
         return self.o_proj.forward(y.view(T, H * dv), allow_parts=not self.whole_output)

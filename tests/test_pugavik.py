@@ -41,7 +41,8 @@ def test_description_names_every_tensor(name):
             d = m["dim"] if m["dim"] == m["vdim"] else -(-max(m["dim"], m["vdim"]) // 16) * 16
             assert need == PagedKV(m["kv_heads"], d, m["mask"]["size"])
         else:
-            assert need == PagedKV(1, -(-(m["kv_rank"] + m["rot_dim"]) // 16) * 16, 0)
+            n = m["kv_rank"] + m["rot_dim"]
+            assert need == PagedKV(1, -(-n // 32) * 32 if n <= 128 else -(-n // 16) * 16, 0)
 
 
 def test_a_looped_model_keeps_a_cache_for_every_pass():

@@ -111,21 +111,28 @@ def test_sigmoid_root_is_stable_at_both_ends():
     _close(got, torch.exp(-torch.nn.functional.softplus(-(z + bias).double()) / 4.0), 1e-6, "with a bias")
 
 
+@pytest.mark.parametrize("page", [32, 64])
 @pytest.mark.parametrize("window", [0, 5, 40, 1000])
 @pytest.mark.parametrize("nh,nkv,d,dv", [(8, 2, 64, 32), (4, 1, 128, 128), (8, 4, 32, 20), (32, 2, 128, 96), (6, 2, 96, 96), (20, 4, 128, 128)])
-def test_matrix_core_headmix_attention_equals_the_plain_kernel(nh, nkv, d, dv, window):
+def test_matrix_core_headmix_attention_equals_the_plain_kernel(nh, nkv, d, dv, window, page):
     """A step with a portion of 19 tokens after 70 cached ones (tiles of 8, 8 and 3 tokens), a decoded token at position 130
-    of another request (pages the window has passed are gone) and a first token of a third: the matrix-core kernel against
-    the plain one on the same cache, and the plain one against the formula."""
+    of another request (pages the window has passed are gone) and a first token of a third: the matrix-core kernel (key
+    tiles of 32 and, on pages of 64, of 64) against the plain one on the same cache, and the plain one against the formula."""
     from infinilm_amd import kernels
     g = torch.Generator().manual_seed(nh * 7 + d + window)
-    page, pages = 32, 12
+    pages = 12
     bf = torch.bfloat16
     kc = torch.randn(pages + 1, nkv, page, d, generator=g).to(bf)
     vc = torch.randn(pages + 1, nkv, d, page, generator=g).to(bf)
     vc[:, :, dv:] = 0
     lens = [89, 131, 1]                                    # keys of each request after this step
-    tables = [[3, 7, 1, -1, -1], [9, 2, 10, 4, 6], [5, -1, -1, -1, -1]]
+    ids = [3, 7, 1, 9, 2, 10, 4, 6, 5]
+    width = -(-131 // page)
+    tables, at = [], 0
+    for n in lens:
+        k = -(-n // page)
+        tables.append(ids[at:at + k] + [-1] * (width - k))
+        at += k
     if 0 < window <= 40:                                   # pages the decoded token's window has passed are given back
         tables[1][:(131 - window) // page] = [-1] * ((131 - window) // page)
     rows_pos = [(0, 70 + i) for i in range(19)] + [(1, 130), (2, 0)]
