@@ -207,11 +207,12 @@ def compare_designs(args) -> dict:
                             share["decay_scan (decay per channel) decode (state read + written / HBM peak)"] = round(64 * 2 * gstate / us(rep_d, "ilm_decay_scan") / HBM_PEAK, 4)
                             share["decay_scan (decay per channel) prefill (4 dk dv flops a token and head / float32 vector peak)"] = round(
                                 4.0 * T * heads * (d // 2) * d / us(rep_p, "ilm_decay_scan") / FLOP_PEAK["fp32"], 4)
-                        if us(rep_d, "ilm_attn_mfma"):   # (the latent layers' attention: one cached row of d entries a token, read as key and as value)
-                            share["latent attention decode (cache read / HBM peak)"] = round(64 * ctx * 2 * d * 2 / us(rep_d, "ilm_attn_mfma") / HBM_PEAK, 4)
-                        if us(rep_p, "ilm_attn_tile"):
+                        lat = "ilm_attn_headmix_mfma (unmixed)"   # (the latent layers' attention: one cached row of d entries a token, read as key and as value)
+                        if us(rep_d, lat):
+                            share["latent attention decode (cache read / HBM peak)"] = round(64 * ctx * 2 * d * 2 / us(rep_d, lat) / HBM_PEAK, 4)
+                        if us(rep_p, lat):
                             share["latent attention prefill (4 d flops a visible key and head / bf16 matrix peak)"] = round(
-                                4.0 * T * T / 2 * heads * d / us(rep_p, "ilm_attn_tile") / FLOP_PEAK["bf16"], 4)
+                                4.0 * T * T / 2 * heads * d / us(rep_p, lat) / FLOP_PEAK["bf16"], 4)
                         if us(rep_p, "ilm_add_layernorm"):
                             share["add_layernorm prefill (stream read + written, two branches read, rows written / HBM peak)"] = round(
                                 T * Hs * (4 + 4 + 2 + 2 + 2) / us(rep_p, "ilm_add_layernorm") / HBM_PEAK, 4)

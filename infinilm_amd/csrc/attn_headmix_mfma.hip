@@ -94,7 +94,10 @@ extern "C" int ilm_headmix_queries(void* qx, const void* q, const void* mix, int
 // ------------------------------------------------------------------------------------------
 // TK: keys a tile (32; tiles of 64 halve the rounds of loads and barriers and measured slower: 437 against 374 us a
 // prompt step at 32 heads of 128, more LDS a workgroup and fewer workgroups a unit)
-template <int D32, int NC, int HPW, int TK>
+// HC (single tokens; one key/value group, or groups of a multiple of 16 heads): the 16 columns of the products are 16 heads of one token instead
+// of 16 tokens of one head (q' of head r in lane r; a wave takes 16 heads, a workgroup 64): a decoded token's keys are then
+// read once for 64 heads instead of once a head.  HPW is 1.
+template <int D32, int NC, int HPW, int TK, bool HC = false>
 __global__ void __launch_bounds__(256)
 attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, const bf16* __restrict__ kc, const bf16* __restrict__ vc,
                          const int* __restrict__ block_tables, const int* __restrict__ seg, const int* __restrict__ pos,
@@ -121,21 +124,22 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
     const int* bt = block_tables + (size_t)seg[t0] * max_blocks;
     const int per = nh / NC;
     // this lane's token (column r of the products)
-    const bool tok_ok = r < ntok;
-    const int tok = t0 + (tok_ok ? r : 0);
-    const int p_tok = p_first + (tok_ok ? r : 0);
+    const bool tok_ok = HC || r < ntok;
+    const int tok = t0 + ((tok_ok && !HC) ? r : 0);
+    const int p_tok = p_first + ((tok_ok && !HC) ? r : 0);
     const int lo_tok = (window > 0 && p_tok - window + 1 > 0) ? p_tok - window + 1 : 0;
     // this wave's heads and their queries
     int head[HPW];
-    bool head_ok[HPW];
+    bool head_ok[HPW], lane_ok[HPW];     // lane_ok: this lane's column holds a head (HC with fewer heads than columns)
     uint4 qf[HPW][NC][D32];
     hx_f32x4 O[HPW][2 * D32];
     float m_run[HPW], l_run[HPW];
 #pragma unroll
     for (int i = 0; i < HPW; ++i) {
-        const int h = (blockIdx.y * 4 + wave) * HPW + i;
-        head_ok[i] = h < nh;
-        head[i] = head_ok[i] ? h : nh - 1;
+        const int h = HC ? (blockIdx.y * 4 + wave) * 16 + r : (blockIdx.y * 4 + wave) * HPW + i;
+        head_ok[i] = HC ? (blockIdx.y * 4 + wave) * 16 < nh : h < nh;     // (uniform over the wave)
+        lane_ok[i] = h < nh;
+        head[i] = h < nh ? h : nh - 1;
         const bf16* qrow = qx + ((size_t)tok * nh + head[i]) * NC * D;
 #pragma unroll
         for (int c = 0; c < NC; ++c)
@@ -249,7 +253,7 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
         l += __shfl_xor(l, 16, 64);
         l += __shfl_xor(l, 32, 64);
         if (chunk_keys > 0) {
-            if (r == 0) {      // (a single token: column 0)
+            if (HC ? lane_ok[i] : r == 0) {      // (a single token: column 0, or every column its head)
                 float* dst = ws + (((size_t)blockIdx.x * gridDim.z + blockIdx.z) * nh + head[i]) * (D + 4);
 #pragma unroll
                 for (int b = 0; b < 2 * D32; ++b)
@@ -260,7 +264,7 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
         }
         if (sink != nullptr) l += __builtin_amdgcn_exp2f(sink[head[i]] * 1.4426950408889634f - m_run[i]);
         const float inv = 1.0f / l;
-        if (tok_ok) {
+        if (tok_ok && lane_ok[i]) {
             bf16* orow = out + (size_t)tok * out_stride + (size_t)head[i] * D;
 #pragma unroll
             for (int b = 0; b < 2 * D32; ++b) {
@@ -304,6 +308,9 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
                                      int n_singles, const void* sink, int nh, int nkv, int d, int page, int max_blocks,
                                      int out_stride, float scale, int window, void* ws, int nz, int chunk_keys,
                                      hipStream_t stream) {
+    // single tokens whose heads come in groups of a multiple of 16: heads as the products' columns
+    // (a block of 16 columns must lie in one key/value group: one group in all, or groups of a multiple of 16 heads)
+    const bool hc = n_tiles == 0 && (nkv == 1 || (nh % 16 == 0 && (nh / (nkv > 0 ? nkv : 1)) % 16 == 0));
     // ws != null (single tokens only): nz chunks of chunk_keys keys a token, float [n_singles][nz][nh][d + 4]
     ILM_REQUIRE(ws == nullptr || (n_tiles == 0 && nz >= 1 && nz <= 65535 && chunk_keys > 0 && chunk_keys % 64 == 0),
                 "attn_headmix_mfma: chunks are for single tokens, in multiples of 64 keys");
@@ -314,16 +321,16 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
                 ((uintptr_t)vc & 15) == 0, "attn_headmix_mfma: rows must be 16-byte / 8-byte aligned");
     const float scale_log2e = scale * 1.4426950408889634f;
 #define HX_LAUNCH(D32_, NC_, HPW_)                                                                                         \
-    HX_LAUNCH_TK(D32_, NC_, HPW_, 32)
-#define HX_LAUNCH_TK(D32_, NC_, HPW_, TK_)                                                                                 \
+    if (hc) HX_LAUNCH_TK(D32_, NC_, 1, 32, true) else HX_LAUNCH_TK(D32_, NC_, HPW_, 32, false)
+#define HX_LAUNCH_TK(D32_, NC_, HPW_, TK_, HC_)                                                                            \
     {                                                                                                                      \
-        auto kern = attn_headmix_mfma_kernel<D32_, NC_, HPW_, TK_>;                                                        \
+        auto kern = attn_headmix_mfma_kernel<D32_, NC_, HPW_, TK_, HC_>;                                                   \
         const int shm = NC_ * TK_ * (D32_ * 32 + 8) * 2 + NC_ * D32_ * 32 * (TK_ + 8) * 2;                                 \
         if (shm > 48 * 1024) {                                                                                             \
             hipError_t e_ = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, shm);       \
             ILM_REQUIRE(e_ == hipSuccess, "attn_headmix_mfma: %d bytes of LDS refused: %s", shm, hipGetErrorString(e_));   \
         }                                                                                                                  \
-        dim3 grid(n_tiles + n_singles, (nh + 4 * HPW_ - 1) / (4 * HPW_), nz);                                              \
+        dim3 grid(n_tiles + n_singles, HC_ ? (nh + 63) / 64 : (nh + 4 * HPW_ - 1) / (4 * HPW_), nz);                       \
         kern<<<grid, 256, shm, stream>>>((bf16*)out, (const bf16*)qx, (const bf16*)kc, (const bf16*)vc,                    \
                                          (const int*)block_tables, (const int*)seg, (const int*)pos, (const int*)tiles,    \
                                          n_tiles, (const int*)singles, (const float*)sink, nh, page, max_blocks,           \

@@ -112,11 +112,12 @@ def _dev(*ts: Optional[torch.Tensor]) -> None:
             raise KernelError("the kernels run on the GPU only; got a CPU tensor")
 
 
-def _run(name: str, *args) -> None:
+def _run(name: str, *args, label: Optional[str] = None) -> None:
+    """`label`: the name the launch's time is filed under, where one entry point serves uses that are worth telling apart."""
     if _TIMES is None:
         rc = getattr(_lib(), name)(*args)
     else:
-        with _timed(name):
+        with _timed(label or name):
             rc = getattr(_lib(), name)(*args)
     if rc != 0:
         raise KernelError(_libmod.last_error())
@@ -1417,6 +1418,8 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                 span = min(span, int(window) + 64)
             hpw = 1 if d > 64 else (2 if nkv == 4 else 4)      # heads a wave, as the kernel's launcher picks them
             passes = -(-nh // (4 * hpw))
+            if nkv == 1 or (nh % 16 == 0 and (nh // nkv) % 16 == 0):   # (heads as the products' columns: 64 heads a workgroup)
+                passes = -(-nh // 64)
             want = max(1, (4 * _num_cus(q.device)) // max(1, bound_rows(n_single) * passes))
             chunk = max(128, -(-(-(-span // want)) // 64) * 64)
             nz = -(-span // chunk)
@@ -1427,7 +1430,7 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         _run("ilm_attn_headmix_mfma", out.data_ptr(), qx.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
              seg_of_token.data_ptr(), positions.data_ptr(), _ptr(tiles) if n_tiles else None, n_tiles, _ptr(rows), n_single,
              _ptr(sink), nh, nkv, d, page, block_tables.shape[1], out.stride(0), float(scale), int(window), _ptr(ws), nz, chunk,
-             _stream())
+             _stream(), label="ilm_attn_headmix_mfma (unmixed)" if mix is None and sink is None else None)
         return out
     _run("ilm_attn_headmix", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
          seg_of_token.data_ptr(), positions.data_ptr(), None, T, _ptr(mix), _ptr(sink), nh, nkv, d, int(dv), page,

@@ -113,11 +113,13 @@ def test_sigmoid_root_is_stable_at_both_ends():
 
 @pytest.mark.parametrize("page", [32, 64])
 @pytest.mark.parametrize("window", [0, 5, 40, 1000])
-@pytest.mark.parametrize("nh,nkv,d,dv", [(8, 2, 64, 32), (4, 1, 128, 128), (8, 4, 32, 20), (32, 2, 128, 96), (6, 2, 96, 96), (20, 4, 128, 128)])
+@pytest.mark.parametrize("nh,nkv,d,dv", [(8, 2, 64, 32), (4, 1, 128, 128), (8, 4, 32, 20), (32, 2, 128, 96), (6, 2, 96, 96), (20, 4, 128, 128),
+                                         (16, 1, 64, 48), (48, 1, 32, 32), (64, 4, 64, 64)])
 def test_matrix_core_headmix_attention_equals_the_plain_kernel(nh, nkv, d, dv, window, page):
     """A step with a portion of 19 tokens after 70 cached ones (tiles of 8, 8 and 3 tokens), a decoded token at position 130
-    of another request (pages the window has passed are gone) and a first token of a third: the matrix-core kernel (key
-    tiles of 32 and, on pages of 64, of 64) against the plain one on the same cache, and the plain one against the formula."""
+    of another request (pages the window has passed are gone) and a first token of a third: the matrix-core kernel against
+    the plain one on the same cache, and the plain one against the formula.  Served by tiles and token by token (where the
+    heads come in groups of 16, 48 or 64 the latter puts heads side by side as the products' columns)."""
     from infinilm_amd import kernels
     g = torch.Generator().manual_seed(nh * 7 + d + window)
     pages = 12
