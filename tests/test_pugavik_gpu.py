@@ -45,7 +45,7 @@ def _close(got, want, tol, what):
 def test_add_layernorm_sums_every_kind_of_addend():
     from infinilm_amd import kernels
     g = torch.Generator().manual_seed(3)
-    for H in (24, 256, 1000, 4100):
+    for H in (24, 250, 256, 1000, 4100):
         r = torch.randn(5, H, generator=g)
         a = torch.randn(5, H, generator=g).to(torch.bfloat16)
         parts = torch.randn(3, 5, H, generator=g)
@@ -503,6 +503,58 @@ def test_logits_do_not_depend_on_the_cut_in_32_bit(case):
     b.step([("r5", toks["r5"][52:130])])
     b.step([("r5", toks["r5"][130:])])
     _close(b.request_logits("r5", 131), a.request_logits("r5", 131), 2e-6, "cut and batched against whole")
+
+
+# ---- random configurations -----------------------------------------------------------------------------------------------
+def _random_config(seed):
+    """Three to five layers of the three kinds in a random order, every size drawn from a short list, a loop over a random
+    stretch (or none), layers without a feed-forward now and then."""
+    import random
+    rnd = random.Random(seed)
+    width = rnd.choice([48, 64, 96, 120, 128])
+    layers = []
+    for _ in range(rnd.randint(3, 5)):
+        kind = rnd.choice(["attention", "latent_attention", "gla"])
+        if kind == "attention":
+            kv = rnd.choice([1, 2, 3, 4])
+            heads = kv * rnd.choice([1, 2, 3])
+            dim = rnd.choice([8, 12, 16, 32, 40, 64])
+            m = P._attention(heads, kv, dim, rnd.choice([dim, 8, 24, 32, 64]), rnd.choice([1, 2, 9, 31, 64, 65, 500]),
+                             rnd.choice([0, 2, dim // 2 // 2 * 2, dim]), base=rnd.choice([100.0, 10000.0, 500000.0]), scale=rnd.choice([0.1, 0.25, dim ** -0.5]))
+        elif kind == "latent_attention":
+            rot = rnd.choice([0, 4, 8, 16, 32])
+            m = P._latent(rnd.choice([1, 2, 3, 4, 8]), rnd.choice([8, 16, 24, 32]), rot, rnd.choice([8, 16, 20, 32]), rnd.choice([16, 24, 48, 96, 112, 136]),
+                          base=rnd.choice([1000.0, 10000.0]))
+        else:
+            m = P._gla(rnd.choice([1, 2, 4]), rnd.choice([8, 16, 20, 32, 64]), rnd.choice([8, 16, 24, 64]), rnd.choice([1.0, 4.0, 16.0]), rnd.choice([2, 4, 7, 16]))
+        layers.append(P._layer(kind, m, rnd.choice([None, 32, 100, 2 * width])))
+    cfg = {"architecture": "Pugavik", "vocab": rnd.choice([50, 131, 640]), "width": width, "embedding": {"scale": rnd.choice([0.5, 1.0, 3.0])},
+           "norm": {"eps": rnd.choice([1e-6, 1e-5])}, "layers": layers}
+    if rnd.random() < 0.7:
+        a = rnd.randrange(len(layers))
+        cfg["loop"] = {"start": a, "stop": rnd.randint(a + 1, len(layers)), "times": rnd.choice([1, 2, 3])}
+    return cfg
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", range(10))
+def test_random_configurations(seed, dtype, tmp_path):
+    """A random configuration, two requests: one whole, one in portions beside the other's decoded tokens, on pages of 16 or
+    64 with four slots; every logit against the plain implementation."""
+    cfg = _random_config(seed)
+    W = make_dir(str(tmp_path), cfg, P.random_weights(cfg, 100 + seed), dtype)
+    ta, tb = tokens(cfg, 75, seed), tokens(cfg, 40, seed + 50)
+    want_a, want_b = P.forward(cfg, W, ta), P.forward(cfg, W, tb)
+    page = 16 if seed % 2 else 64
+    drv = Driver(str(tmp_path), dtype, num_pages=-(-75 // page) + -(-40 // page) + 1, page_size=page, max_requests=4)
+    drv.step([("a", ta[:33])])
+    drv.step([("a", ta[33:35]), ("b", tb[:19])])
+    drv.step([("a", ta[35:70]), ("b", tb[19:20])])
+    for i in range(5):
+        drv.step([("a", ta[70 + i:71 + i]), ("b", tb[20 + 4 * i:24 + 4 * i])])
+    tol = lambda t, want: TOL[dtype] if dtype == "float32" else max(TOL[dtype], 2.0 * rel_err(P.forward(cfg, W, t, round_to=torch.bfloat16), want))
+    ea, eb = rel_err(drv.request_logits("a", 75), want_a), rel_err(drv.request_logits("b", 40), want_b)
+    assert ea < tol(ta, want_a) and eb < tol(tb, want_b), f"seed {seed}: {ea:.3e}, {eb:.3e}; {json.dumps(cfg)}"
 
 
 # ---- the entry point and its scheduler ------------------------------------------------------------------------------------
