@@ -26,7 +26,6 @@
 typedef __attribute__((ext_vector_type(8))) __bf16 hx_bf16x8;
 typedef __attribute__((ext_vector_type(4))) float hx_f32x4;
 
-#define HX_TT 8            // tokens a tile at most (the step's lists hold tiles of up to 8)
 #define HX_NEG (-1.0e30f)
 
 __device__ __forceinline__ hx_f32x4 hx_mfma(uint4 a, uint4 b, hx_f32x4 c) {
@@ -103,7 +102,7 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
                          const int* __restrict__ block_tables, const int* __restrict__ seg, const int* __restrict__ pos,
                          const int* __restrict__ tiles, int n_tiles, const int* __restrict__ singles,
                          const float* __restrict__ sink, int nh, int page, int max_blocks, int out_stride, float scale_log2e,
-                         int window, float* __restrict__ ws, int chunk_keys) {
+                         int window, float* __restrict__ ws, int chunk_keys, const int* __restrict__ seg_offsets) {
     constexpr int D = D32 * 32, KROW = D + 8, VROW = TK + 8, NS = TK / 16, NP = TK / 32;
     extern __shared__ __attribute__((aligned(16))) unsigned char hx_smem[];
     bf16* Ks = reinterpret_cast<bf16*>(hx_smem);                 // [NC][32][KROW]
@@ -113,6 +112,14 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
     if ((int)blockIdx.x < n_tiles) {
         t0 = tiles[2 * blockIdx.x];
         ntok = tiles[2 * blockIdx.x + 1];
+        // The step's lists hold tiles of up to 8 tokens, cut from each request's first row on.  With the requests' first
+        // rows at hand two neighbours make one tile of 16 (all the products' columns): the even tiles of a request take
+        // their successors' tokens along, the odd ones leave.
+        if (seg_offsets != nullptr && ntok > 0) {
+            const int sg = seg[t0], first = seg_offsets[sg], end = seg_offsets[sg + 1];
+            if (((t0 - first) >> 3) & 1) return;
+            ntok = min(16, end - t0);
+        }
     } else {
         const int i = blockIdx.x - n_tiles;
         t0 = singles != nullptr ? singles[i] : i;
@@ -159,23 +166,46 @@ attn_headmix_mfma_kernel(bf16* __restrict__ out, const bf16* __restrict__ qx, co
         kb_begin += blockIdx.z * chunk_keys;
         kb_end = min(p_last, kb_begin + chunk_keys - 1);
     }
-    for (int kb = kb_begin; kb <= kb_end; kb += TK) {
+    // A tile is on its way from the cache into registers while the tile before it is multiplied: a workgroup's tiles are a
+    // chain (load, barrier, multiply), and with one head a wave the chain's length, not the chip's throughput, sets the time
+    // of a long request's last tiles.
+    constexpr int KPER = (KPIECES + 255) / 256, VPER = (VPIECES + 255) / 256;
+    uint4 kreg[KPER], vreg[VPER];
+    auto fetch = [&](int kb) {
         const int pg = bt[kb / page];                            // (a tile lies on one page: the page size is a multiple of 32)
-        const int off = kb % page;
-        __syncthreads();                                         // the tile before this one has been read by every wave
-        for (int pc = tid; pc < KPIECES; pc += 256) {
+        const int off = kb % page;                               // pg < 0: a page the window has passed; its keys weigh nothing
+#pragma unroll
+        for (int i = 0; i < KPER; ++i) {
+            const int pc = tid + i * 256;
             const int c = pc / (TK * (D / 8)), rest = pc % (TK * (D / 8)), key = rest / (D / 8), piece = rest % (D / 8);
-            uint4 v = zero4;
-            if (pg >= 0) v = *reinterpret_cast<const uint4*>(kc + (((size_t)pg * NC + c) * page + off + key) * D + piece * 8);
-            *reinterpret_cast<uint4*>(Ks + (c * TK + key) * KROW + piece * 8) = v;
+            kreg[i] = zero4;
+            if (pc < KPIECES && pg >= 0) kreg[i] = *reinterpret_cast<const uint4*>(kc + (((size_t)pg * NC + c) * page + off + key) * D + piece * 8);
         }
-        for (int pc = tid; pc < VPIECES; pc += 256) {
+#pragma unroll
+        for (int i = 0; i < VPER; ++i) {
+            const int pc = tid + i * 256;
             const int c = pc / (D * (TK / 8)), rest = pc % (D * (TK / 8)), row = rest / (TK / 8), piece = rest % (TK / 8);
-            uint4 v = zero4;
-            if (pg >= 0) v = *reinterpret_cast<const uint4*>(vc + (((size_t)pg * NC + c) * D + row) * page + off + piece * 8);
-            *reinterpret_cast<uint4*>(Vs + (c * D + row) * VROW + piece * 8) = v;
+            vreg[i] = zero4;
+            if (pc < VPIECES && pg >= 0) vreg[i] = *reinterpret_cast<const uint4*>(vc + (((size_t)pg * NC + c) * D + row) * page + off + piece * 8);
+        }
+    };
+    if (kb_begin <= kb_end) fetch(kb_begin);
+    for (int kb = kb_begin; kb <= kb_end; kb += TK) {
+        __syncthreads();                                         // the tile before this one has been read by every wave
+#pragma unroll
+        for (int i = 0; i < KPER; ++i) {
+            const int pc = tid + i * 256;
+            const int c = pc / (TK * (D / 8)), rest = pc % (TK * (D / 8)), key = rest / (D / 8), piece = rest % (D / 8);
+            if (pc < KPIECES) *reinterpret_cast<uint4*>(Ks + (c * TK + key) * KROW + piece * 8) = kreg[i];
+        }
+#pragma unroll
+        for (int i = 0; i < VPER; ++i) {
+            const int pc = tid + i * 256;
+            const int c = pc / (D * (TK / 8)), rest = pc % (D * (TK / 8)), row = rest / (TK / 8), piece = rest % (TK / 8);
+            if (pc < VPIECES) *reinterpret_cast<uint4*>(Vs + (c * D + row) * VROW + piece * 8) = vreg[i];
         }
         __syncthreads();
+        if (kb + TK <= kb_end) fetch(kb + TK);
         // head by head (a version that read every key and value fragment from LDS once for all heads of a wave kept more
         // registers live and measured slower: 455 against 374 us a prompt step at 32 heads of 128)
 #pragma unroll
@@ -302,12 +332,14 @@ extern "C" int ilm_attn_headmix_mfma_ok(int nh, int nkv, int d, int page) {
 }
 
 // qx [T, nh, nkv, d] from ilm_headmix_queries; tiles [n_tiles, 2] = (first row, count <= 8) and n_singles single rows
-// (`singles` null: rows 0 .. n_singles - 1; an entry -1 or a count 0 names nothing)
+// (`singles` null: rows 0 .. n_singles - 1; an entry -1 or a count 0 names nothing); seg_offsets (may be null): the first row
+// of every request of the step and the end of the last, with which tiles cut 8 by 8 from a request's first row are served
+// two at a time
 extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, const void* vc, const void* block_tables,
                                      const void* seg, const void* pos, const void* tiles, int n_tiles, const void* singles,
                                      int n_singles, const void* sink, int nh, int nkv, int d, int page, int max_blocks,
                                      int out_stride, float scale, int window, void* ws, int nz, int chunk_keys,
-                                     hipStream_t stream) {
+                                     const void* seg_offsets, hipStream_t stream) {
     // single tokens whose heads come in groups of a multiple of 16: heads as the products' columns
     // (a block of 16 columns must lie in one key/value group: one group in all, or groups of a multiple of 16 heads)
     const bool hc = n_tiles == 0 && (nkv == 1 || (nh % 16 == 0 && (nh / (nkv > 0 ? nkv : 1)) % 16 == 0));
@@ -334,7 +366,8 @@ extern "C" int ilm_attn_headmix_mfma(void* out, const void* qx, const void* kc, 
         kern<<<grid, 256, shm, stream>>>((bf16*)out, (const bf16*)qx, (const bf16*)kc, (const bf16*)vc,                    \
                                          (const int*)block_tables, (const int*)seg, (const int*)pos, (const int*)tiles,    \
                                          n_tiles, (const int*)singles, (const float*)sink, nh, page, max_blocks,           \
-                                         out_stride, scale_log2e, window, (float*)ws, chunk_keys);                         \
+                                         out_stride, scale_log2e, window, (float*)ws, chunk_keys,                          \
+                                         (const int*)seg_offsets);                                                         \
     }
 #define HX_BY_NC(D32_)                                                      \
     switch (nkv) {                                                          \

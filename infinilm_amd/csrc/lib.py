@@ -58,7 +58,7 @@ _SIGNATURES = {
     "ilm_qkv_norm_rope_kvwrite": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
     "ilm_attn_headmix": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ilm_headmix_queries": [_P, _P, _P, _I, _I, _I, _I, _I, _P],
-    "ilm_attn_headmix_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _I, _I, _P],
+    "ilm_attn_headmix_mfma": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _I, _I, _P, _P],
     "ilm_latent_prep": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P],
     "ilm_head_gemm": [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _L, _I, _I, _P],
     "ilm_group_norm_gate": [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _I, _I, _I, _L, _P],

@@ -1365,7 +1365,7 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       seg_of_token: torch.Tensor, positions: torch.Tensor, nh: int, nkv: int, d: int, dv: int, scale: float,
                       window: int = 0, mix: Optional[torch.Tensor] = None, sink: Optional[torch.Tensor] = None,
                       tiles: Optional[torch.Tensor] = None, single_rows: Optional[torch.Tensor] = None,
-                      max_total_len: Optional[int] = None) -> torch.Tensor:
+                      max_total_len: Optional[int] = None, seg_offsets: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Attention of every token over its request's cached keys (its last `window` positions, or all) where the scaled
     scores of the heads are mixed before the softmax, s_h = sum_g mix[h, g] raw_g (`mix` float32 [nh, nh] or None),
     and every head's denominator holds one more term exp(sink[h]) (`sink` float32 [nh] or None); with neither it is the
@@ -1373,7 +1373,9 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     tables as for `paged_attention`; `dv`: the entries of a value head that count.  `tiles` [n, 2] = (first row, count <=
     ATT_TILE_TOKENS) lists runs of consecutive tokens of one request and `single_rows` the remaining rows (without them
     every token is served on its own); the matrix-core kernel (bfloat16, heads of 32 to 128 in steps of 32, 1, 2 or 4
-    key/value groups, pages of a multiple of 32) works by them, the plain kernel token by token.  Returns [T, nh*d]."""
+    key/value groups, pages of a multiple of 32) works by them, the plain kernel token by token.  `seg_offsets` (the step's
+    first row of every request, and the end of the last): tiles that were cut 8 by 8 from each request's first row are then
+    served two at a time.  Returns [T, nh*d]."""
     _dev(q, k_cache, v_cache, block_tables, seg_of_token, positions, mix, sink)
     _i32(block_tables, "block_tables")
     _i32(seg_of_token, "seg_of_token")
@@ -1400,6 +1402,9 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
             qx = torch.empty((T, nh, nkv, d), dtype=BF16, device=q.device)
             _run("ilm_headmix_queries", qx.data_ptr(), q.data_ptr(), _ptr(mix), T, nh, nkv, d, q.stride(0), _stream())
         n_tiles, n_single, rows = 0, T, None
+        if seg_offsets is not None:
+            _dev(seg_offsets)
+            _i32(seg_offsets, "seg_offsets")
         if tiles is not None and tiles.numel() > 0:
             _i32(tiles, "tiles")
             n_tiles, n_single = tiles.numel() // 2, 0
@@ -1430,7 +1435,7 @@ def headmix_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
         _run("ilm_attn_headmix_mfma", out.data_ptr(), qx.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
              seg_of_token.data_ptr(), positions.data_ptr(), _ptr(tiles) if n_tiles else None, n_tiles, _ptr(rows), n_single,
              _ptr(sink), nh, nkv, d, page, block_tables.shape[1], out.stride(0), float(scale), int(window), _ptr(ws), nz, chunk,
-             _stream(), label="ilm_attn_headmix_mfma (unmixed)" if mix is None and sink is None else None)
+             _ptr(seg_offsets) if n_tiles else None, _stream(), label="ilm_attn_headmix_mfma (unmixed)" if mix is None and sink is None else None)
         return out
     _run("ilm_attn_headmix", out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
          seg_of_token.data_ptr(), positions.data_ptr(), None, T, _ptr(mix), _ptr(sink), nh, nkv, d, int(dv), page,

@@ -105,7 +105,8 @@ class GQAttention(Mixer):
             o = kernels.headmix_attention(qkv, cache_view.k, cache_view.v, cache_view.block_tables, batch.seg_of_token,
                                           batch.positions, self.nh, self.nkv, self.d, self.dv, self.scale, self.window,
                                           mix=self.head_mix, sink=self.sink, tiles=batch.att_tiles,
-                                          single_rows=batch.att_single_rows, max_total_len=batch.max_total_len)
+                                          single_rows=batch.att_single_rows, max_total_len=batch.max_total_len,
+                                          seg_offsets=batch.seg_offsets)
         else:
             o = self._plain_attention(qkv, batch, cache_view)
         if tail is not None:   # the output projection adds into the residual stream itself, where its kernel can

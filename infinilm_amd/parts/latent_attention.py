@@ -78,7 +78,7 @@ class LatentAttention(Mixer):
         if rows.dtype == torch.bfloat16 and kernels.headmix_mfma_ok(H, 1, d, view.page_size, rows.dtype):
             o = kernels.headmix_attention(q2, view.k, view.v, view.block_tables, batch.seg_of_token, batch.positions, H, 1, d, rank,
                                           self.scale, self.window, tiles=batch.att_tiles, single_rows=batch.att_single_rows,
-                                          max_total_len=batch.max_total_len)
+                                          max_total_len=batch.max_total_len, seg_offsets=batch.seg_offsets)
         else:
             o = kernels.paged_attention(q2, view.k, view.v, view.block_tables, batch.seg_of_token, batch.positions, H, 1, d,
                                         self.scale, self.window, batch.max_total_len, batch.att_tiles, batch.att_single_rows,

@@ -147,6 +147,8 @@ def test_matrix_core_headmix_attention_equals_the_plain_kernel(nh, nkv, d, dv, w
             d ** -0.5, window)
     tiles, singles = i32([[0, 8], [8, 8], [16, 3], [0, 0]]), i32([19, -1, 20])
     fast = kernels.headmix_attention(*args, mix=mix.to(DEV), sink=sink.to(DEV), tiles=tiles, single_rows=singles).cpu()
+    paired = kernels.headmix_attention(*args, mix=mix.to(DEV), sink=sink.to(DEV), tiles=tiles, single_rows=singles,
+                                       seg_offsets=i32([0, 19, 20, 21])).cpu()
     each = kernels.headmix_attention(*args, mix=mix.to(DEV), sink=sink.to(DEV)).cpu()
     old = kernels.USE_HEADMIX_MFMA
     kernels.USE_HEADMIX_MFMA = False
@@ -169,6 +171,7 @@ def test_matrix_core_headmix_attention_equals_the_plain_kernel(nh, nkv, d, dv, w
         want[t] = torch.stack([prob[h] @ vals[:, h // per] for h in range(nh)])
     _close(plain.view(T, nh, d), want, 1e-2, "the plain kernel against the formula")
     _close(fast.view(T, nh, d), want, 2e-2, "the matrix-core kernel, by tiles")
+    _close(paired.view(T, nh, d), want, 2e-2, "the matrix-core kernel, tiles two at a time")
     _close(each.view(T, nh, d), want, 2e-2, "the matrix-core kernel, token by token")
 
 
