@@ -8,8 +8,9 @@
 // exp(sink_h) in the denominator.  Cost of the score product: C times that of unmixed heads, and no exchange of scores
 // between heads; for many groups the plain kernel's explicit mixing does less work.
 //
-// A workgroup = one item (a tile of up to 8 consecutive tokens of a request, or a single token) x one pass of 4 HPW
-// heads; its 4 waves take HPW heads each.  Keys go by in tiles of 32 or 64 aligned to the absolute key index; K [group][key][d]
+// A workgroup = one item (a tile of up to 16 consecutive tokens of a request, or a single token) x one pass of 4 HPW
+// heads; its 4 waves take HPW heads each (for single tokens, where the groups allow it, 16 heads each: the heads are then
+// the products' columns in place of the tokens).  Keys go by in tiles of 32 aligned to the absolute key index; K [group][key][d]
 // and V [group][d][key] of a tile pass through LDS once for all heads of the pass.  Per head and tile:
 //   S^T [keys x 16 tokens] = K q'^T           (v_mfma_f32_16x16x32_bf16: A = K rows, B = q' rows; lane (r, g4) gets
 //                                              keys 4 g4 .. 4 g4 + 3 of each 16-key half for token r)
